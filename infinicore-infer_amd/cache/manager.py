@@ -37,6 +37,8 @@ class GroupSpec:
     window: Optional[int] = None
     slots: tuple = ()                   # cache slot ids (positions in the model's cache list)
     planes: int = 2                     # tensors per slot (keys and values: 2; one latent per token: 1)
+    plane_dims: tuple = ()              # width of each plane when they differ; empty: all head_dim
+    keep_first: int = 0                 # 'window': the first tokens that stay readable for good
 
     def __post_init__(self):
         if self.kind not in ("full", "window"):
@@ -45,6 +47,14 @@ class GroupSpec:
             raise CacheError("a window group needs a positive window")
         if self.planes <= 0:
             raise CacheError("a group needs at least one plane")
+        if self.plane_dims and len(self.plane_dims) != self.planes:
+            raise CacheError("plane_dims names one width per plane")
+        if self.keep_first < 0:
+            raise CacheError("keep_first must not be negative")
+
+    def dims(self) -> tuple:
+        """Width of every plane."""
+        return tuple(self.plane_dims) if self.plane_dims else (self.head_dim,) * self.planes
 
 
 class PagePool:
@@ -86,7 +96,7 @@ class RequestEntry:
     state_slot: int
     length: int = 0                                  # tokens whose keys are in the cache
     tables: List[List[int]] = field(default_factory=list)   # per group: page id per logical page, -1 = given back
-    first_live: List[int] = field(default_factory=list)     # per group: first logical page still held
+    first_live: List[int] = field(default_factory=list)     # per group: pages below it are given back (but for a window's kept first pages)
     serial: int = 0                                  # admission number: tells two lives of one request id apart
 
 
@@ -233,9 +243,10 @@ class CacheManager:
             if spec.kind != "window":
                 continue
             # the next query sits at position e.length and reads keys > e.length - window
-            dead_keys = e.length - spec.window + 1            # keys < dead_keys are never read again
+            dead_keys = e.length - spec.window + 1            # keys < dead_keys are never read again ..
             dead_pages = max(0, dead_keys // self.page_size)
-            for j in range(e.first_live[g], min(dead_pages, len(e.tables[g]))):
+            kept_pages = self._pages_for(spec.keep_first)     # .. but for the first keep_first keys: their pages stay
+            for j in range(max(e.first_live[g], kept_pages), min(dead_pages, len(e.tables[g]))):
                 self.pools[g].free(e.tables[g][j])
                 e.tables[g][j] = -1
                 n += 1

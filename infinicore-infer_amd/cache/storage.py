@@ -6,6 +6,8 @@ Layout of one plane of a cache slot (one attention layer's keys or values):
 page are one contiguous run, which is what the attention kernels stream.
 A group holds ``[n_slots, planes, num_pages, n_kv_heads, page_size, head_dim]``;
 attention has two planes (K, V), a mixer that caches one vector per token has one.
+When a group's planes differ in width (keys of 64, values of 32 entries per head) it
+holds one tensor ``[n_slots, 1, num_pages, n_kv_heads, page_size, width]`` per plane.
 """
 from typing import Dict, List, Sequence, Tuple
 
@@ -23,8 +25,14 @@ class CacheStorage:
         self.group_planes: List[torch.Tensor] = []
         self._slot_index: Dict[int, Tuple[int, int]] = {}      # cache slot -> (group, index in group)
         for g, spec in enumerate(groups):
-            planes = torch.empty((len(spec.slots), spec.planes, num_pages[g], spec.n_kv_heads, page_size, spec.head_dim),
-                                 dtype=dtype, device=device)
+            dims = spec.dims()
+            if len(set(dims)) == 1:
+                planes = torch.empty((len(spec.slots), spec.planes, num_pages[g], spec.n_kv_heads, page_size, dims[0]),
+                                     dtype=dtype, device=device)
+            else:
+                # planes of different widths (keys wider than values): one tensor per plane, [slots, 1, pages, ..]
+                planes = tuple(torch.empty((len(spec.slots), 1, num_pages[g], spec.n_kv_heads, page_size, w),
+                                           dtype=dtype, device=device) for w in dims)
             self.group_planes.append(planes)
             for i, s in enumerate(spec.slots):
                 self._slot_index[s] = (g, i)
@@ -46,7 +54,12 @@ class CacheStorage:
         views = self._kv_views.get(slot)
         if views is None:
             g, i = self._slot_index[slot]
-            views = self._kv_views[slot] = tuple(self.group_planes[g][i, j] for j in range(self.group_planes[g].shape[1]))
+            gp = self.group_planes[g]
+            if isinstance(gp, tuple):
+                views = tuple(p[i, 0] for p in gp)
+            else:
+                views = tuple(gp[i, j] for j in range(gp.shape[1]))
+            self._kv_views[slot] = views
         return views
 
     def kv(self, slot: int):
@@ -73,7 +86,8 @@ class CacheStorage:
         host[0, :n] = torch.as_tensor(list(src_pages), dtype=torch.int32)
         host[1, :n] = torch.as_tensor(list(dst_pages), dtype=torch.int32)
         dev.copy_(host, non_blocking=True)
-        ops.copy_pages(planes, dev[0, :n], dev[1, :n])
+        for p in (planes if isinstance(planes, tuple) else (planes,)):
+            ops.copy_pages(p, dev[0, :n], dev[1, :n])
 
     def copy_state(self, src_slot: int, dst_slot: int) -> None:
         for t in self.state.values():
@@ -84,5 +98,5 @@ class CacheStorage:
             t[state_slot].zero_()
 
     def bytes(self) -> int:
-        n = sum(p.numel() * p.element_size() for p in self.group_planes)
+        n = sum(p.numel() * p.element_size() for gp in self.group_planes for p in (gp if isinstance(gp, tuple) else (gp,)))
         return n + sum(t.numel() * t.element_size() for t in self.state.values())

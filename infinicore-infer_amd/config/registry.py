@@ -37,11 +37,13 @@ def registered_architectures():
 
 
 def resolve_architecture(config: dict) -> type:
-    """Look the architecture up by ``model_type`` first, then by each entry of
+    """Look the architecture up by ``model_type`` first, then by ``architecture`` and each entry of
     ``architectures``."""
     keys = []
     if "model_type" in config:
         keys.append(config["model_type"])
+    if isinstance(config.get("architecture"), str):
+        keys.append(config["architecture"])
     keys.extend(config.get("architectures") or [])
     for k in keys:
         if k in _ARCHITECTURES:

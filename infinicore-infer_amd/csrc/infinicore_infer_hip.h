@@ -65,6 +65,23 @@ int ic_attn_prefill_parts(int n_tiles, int nh, int dh, int max_keys, int compute
 int ic_attn_prefill_parts_of_step(int dtype, int n_tiles, int nh, int dh, int max_position, int window, int compute_units, int* part_len);   // max_keys from the step's largest position and the window
 int ic_attn_prefill_split(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, int groups, int parts, int part_len, float* scratch, long long scratch_floats, int* counters, hipStream_t stream);
 
+// ---- stream_rows.hip: decoders whose sublayers read the residual stream and are normalised on the way back ----------
+// x[t, 2i] = table[tok, 2i] * scale + sin(p f_i), x[t, 2i+1] = .. + cos(p f_i) (freq: float32 [d/2]); copy (nullable): x in copy_dtype.
+int ic_embed_sinusoid(const int* tokens, const int* positions, const void* table, int table_dtype, const float* freq, float* x, void* copy, int copy_dtype, int T, int d, float scale, hipStream_t stream);
+// x[t] += rmsnorm(y[t] + bias) * w (bias nullable, w float32 [d]); copy (nullable): the new x in copy_dtype.
+int ic_norm_into_stream(const void* y, int y_dtype, const float* bias, const float* w, float* x, void* copy, int copy_dtype, int T, int d, float eps, hipStream_t stream);
+// A token's projected row [q | k | v | ..]: bias, query/key norm (norm_mode 0 none, 1 per head with w[dk], 2 whole row with w[nh dk] / w[nkvh dk]),
+// value mixing (mix_mode 0 none, 1 keep v in v_keep float32 [T, nkvh dv], 2 v = (1 - lambda[0]) v + lambda[0] v_keep), q to q_out [T, nh dk],
+// k and v to the cache planes at slots[t] (K [pages, nkvh, page_size, dk], V [.., dv]).
+int ic_qk_norm_store(const void* rows, int row_stride, int dtype, const float* bias, const float* qw, const float* kw, int norm_mode, float eps, int mix_mode, const float* lambda, float* v_keep, void* q_out, void* kcache, void* vcache, const int* slots, int T, int nh, int nkvh, int dk, int dv, int page_size, hipStream_t stream);
+// out = act(in) element by element; kind 0: relu(z)^2, 1: gelu_tanh(z), 2: silu(z).
+int ic_activation(const void* in, void* out, int dtype, long long n, int kind, hipStream_t stream);
+
+// ---- attn_span.hip: keys and values of different sizes, a window plus kept first keys, a sink, an output gate --------
+// Query at position i sees key j when j <= i and (window == 0 or i - j < window or j < keep_first); sink: 1 joins the
+// softmax's denominator; gate (nullable): out *= sigmoid(gate[t, h dv + d]).
+int ic_attn_span_generic(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* token_req, const int* positions, int T, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, hipStream_t stream);
+
 // ---- gemm.hip ---------------------------------------------------------------------------------------
 // A norm y = x * rsqrt(mean(x^2) + eps) * w between two products of M <= 16 rows can be split over them: the
 // product before it adds its result to the residual stream, stores x * w and the sums of x^2 per row and

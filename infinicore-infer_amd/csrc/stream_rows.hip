@@ -1,0 +1,238 @@
+// Row kernels of decoders that normalise a sublayer's OUTPUT before it joins the residual stream
+// (x += norm(f(x))) and whose sublayers read the stream itself:
+//   * embedding gather with a sinusoidal position vector added,
+//   * x += rmsnorm(y + bias) * w, with the stream's copy in the compute dtype written along,
+//   * bias, query/key norm (per head or over the whole row), value mixing with an earlier layer's
+//     values and the write of keys and values into the paged cache, in one pass over a token's
+//     projected row,
+//   * element-wise activations of a dense feed-forward.
+// The residual stream is float32; every norm, sum of squares, angle and mix is float32.
+//
+// Cache layout of one layer: K plane [num_pages, n_kv_heads, page_size, key_dim], V plane
+// [num_pages, n_kv_heads, page_size, value_dim].
+#include "common.h"
+
+// ---------------------------------------------------------------------------------------------
+// x[t, 2i] = table[tok, 2i] * scale + sin(p f_i), x[t, 2i+1] = table[tok, 2i+1] * scale + cos(p f_i);
+// f_i is a float32 table [d/2] made by the host; the angle is the float32 product p * f_i.
+// copy (nullable): x rounded to the compute dtype.
+// ---------------------------------------------------------------------------------------------
+template <typename TW, typename TC>
+__global__ void embed_sinusoid_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
+                                      const TW* __restrict__ table, const float* __restrict__ freq,
+                                      float* __restrict__ x, TC* __restrict__ copy, int d, float scale) {
+    const int t = blockIdx.x;
+    const TW* row = table + (size_t)tokens[t] * d;
+    const float p = (float)positions[t];
+    float* o = x + (size_t)t * d;
+    for (int i = threadIdx.x; i < d / 2; i += blockDim.x) {
+        const float ang = p * freq[i];
+        const float a = to_f32(row[2 * i]) * scale + sinf(ang);
+        const float b = to_f32(row[2 * i + 1]) * scale + cosf(ang);
+        o[2 * i] = a;
+        o[2 * i + 1] = b;
+        if (copy) {
+            copy[(size_t)t * d + 2 * i] = from_f32<TC>(a);
+            copy[(size_t)t * d + 2 * i + 1] = from_f32<TC>(b);
+        }
+    }
+}
+
+IC_EXPORT int ic_embed_sinusoid(const int* tokens, const int* positions, const void* table, int table_dtype,
+                                const float* freq, float* x, void* copy, int copy_dtype, int T, int d, float scale,
+                                hipStream_t stream) {
+    if (T <= 0) return IC_OK;
+    if (d <= 0 || (d & 1)) return IC_ERR_ARG;
+    dim3 grid(T), block(256);
+    if (table_dtype == IC_F32 && (copy == nullptr || copy_dtype == IC_F32))
+        hipLaunchKernelGGL((embed_sinusoid_kernel<float, float>), grid, block, 0, stream, tokens, positions,
+                           (const float*)table, freq, x, (float*)copy, d, scale);
+    else if (table_dtype == IC_BF16 && (copy == nullptr || copy_dtype == IC_BF16))
+        hipLaunchKernelGGL((embed_sinusoid_kernel<bf16, bf16>), grid, block, 0, stream, tokens, positions,
+                           (const bf16*)table, freq, x, (bf16*)copy, d, scale);
+    else if (table_dtype == IC_F32 && copy_dtype == IC_BF16)
+        hipLaunchKernelGGL((embed_sinusoid_kernel<float, bf16>), grid, block, 0, stream, tokens, positions,
+                           (const float*)table, freq, x, (bf16*)copy, d, scale);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// x[t] += (y[t] + bias) * rsqrt(mean((y[t] + bias)^2) + eps) * w;  copy[t] = x[t] in the compute dtype.
+// One block per row; the row is read twice (the second time from cache).
+// ---------------------------------------------------------------------------------------------
+template <typename TY, typename TC>
+__global__ void __launch_bounds__(256)
+norm_into_stream_kernel(const TY* __restrict__ y, const float* __restrict__ bias, const float* __restrict__ w,
+                        float* __restrict__ x, TC* __restrict__ copy, int d, float eps) {
+    __shared__ float red[16];
+    const int t = blockIdx.x;
+    const TY* yr = y + (size_t)t * d;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = to_f32(yr[i]) + (bias ? bias[i] : 0.f);
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float r = 1.0f / sqrtf(ss / (float)d + eps);
+    float* xr = x + (size_t)t * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) {
+        const float v = to_f32(yr[i]) + (bias ? bias[i] : 0.f);
+        const float s = xr[i] + v * r * w[i];
+        xr[i] = s;
+        if (copy) copy[(size_t)t * d + i] = from_f32<TC>(s);
+    }
+}
+
+IC_EXPORT int ic_norm_into_stream(const void* y, int y_dtype, const float* bias, const float* w, float* x, void* copy,
+                                  int copy_dtype, int T, int d, float eps, hipStream_t stream) {
+    if (T <= 0) return IC_OK;
+    if (d <= 0) return IC_ERR_ARG;
+    dim3 grid(T), block(256);
+    if (y_dtype == IC_F32 && (copy == nullptr || copy_dtype == IC_F32))
+        hipLaunchKernelGGL((norm_into_stream_kernel<float, float>), grid, block, 0, stream, (const float*)y, bias, w, x,
+                           (float*)copy, d, eps);
+    else if (y_dtype == IC_BF16 && (copy == nullptr || copy_dtype == IC_BF16))
+        hipLaunchKernelGGL((norm_into_stream_kernel<bf16, bf16>), grid, block, 0, stream, (const bf16*)y, bias, w, x,
+                           (bf16*)copy, d, eps);
+    else if (y_dtype == IC_F32 && copy_dtype == IC_BF16)
+        hipLaunchKernelGGL((norm_into_stream_kernel<float, bf16>), grid, block, 0, stream, (const float*)y, bias, w, x,
+                           (bf16*)copy, d, eps);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// One token's projected row [q (nh * dk) | k (nkvh * dk) | v (nkvh * dv) | ...] of row_stride elements:
+//   q <- norm(q + bq) -> q_out[t] (compute dtype, row stride nh * dk)
+//   k <- norm(k + bk) -> K plane at slots[t]
+//   v <- v + bv; mix_mode 1: v_keep[t] = v (float32, for later layers of this step);
+//                mix_mode 2: v = (1 - lambda) v + lambda v_keep[t]        -> V plane at slots[t]
+// norm_mode 0: none; 1: every head's dk entries to unit root mean square, times w[dk] (shared by the heads);
+// 2: the whole of q (or k) to unit root mean square, times w[nh * dk] (or w[nkvh * dk]).
+// One block per token, the row in LDS as float32 (dynamic, (nh + nkvh) * dk + nkvh * dv floats).
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_store_kernel(const T* __restrict__ rows, int row_stride, const float* __restrict__ bias,
+                     const float* __restrict__ qw, const float* __restrict__ kw, int norm_mode, float eps,
+                     int mix_mode, const float* __restrict__ lambda, float* __restrict__ v_keep,
+                     T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache,
+                     const int* __restrict__ slots, int nh, int nkvh, int dk, int dv, int page_size) {
+    extern __shared__ float row[];
+    __shared__ float red[16];
+    __shared__ float head_r[512];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int nq = nh * dk, nk = nkvh * dk, nv = nkvh * dv, n = nq + nk + nv;
+    const T* src = rows + (size_t)t * row_stride;
+    for (int i = tid; i < n; i += blockDim.x) row[i] = to_f32(src[i]) + (bias ? bias[i] : 0.f);
+    __syncthreads();
+    const int slot = slots ? slots[t] : -1;
+    const int pg = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - pg * page_size : 0;
+
+    if (norm_mode == 1) {
+        // one wave per head, heads of q and k alike
+        const int lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+        for (int h = wave; h < nh + nkvh; h += nw) {
+            float ss = 0.f;
+            for (int j = lane; j < dk; j += 64) { const float v = row[h * dk + j]; ss += v * v; }
+            ss = wave_sum(ss);
+            if (lane == 0) head_r[h] = 1.0f / sqrtf(ss / (float)dk + eps);
+        }
+        __syncthreads();
+        for (int i = tid; i < nq + nk; i += blockDim.x) {
+            const int h = i / dk, j = i - h * dk;
+            row[i] = row[i] * head_r[h] * (h < nh ? qw[j] : kw[j]);
+        }
+    } else if (norm_mode == 2) {
+        float sq = 0.f, sk = 0.f;
+        for (int i = tid; i < nq; i += blockDim.x) sq += row[i] * row[i];
+        for (int i = nq + tid; i < nq + nk; i += blockDim.x) sk += row[i] * row[i];
+        sq = block_sum(sq, red);
+        sk = block_sum(sk, red);
+        const float rq = 1.0f / sqrtf(sq / (float)nq + eps), rk = 1.0f / sqrtf(sk / (float)nk + eps);
+        for (int i = tid; i < nq; i += blockDim.x) row[i] = row[i] * rq * qw[i];
+        for (int i = tid; i < nk; i += blockDim.x) row[nq + i] = row[nq + i] * rk * kw[i];
+    }
+    __syncthreads();
+    for (int i = tid; i < nq; i += blockDim.x) q_out[(size_t)t * nq + i] = from_f32<T>(row[i]);
+    if (slot >= 0 && kcache) {
+        for (int i = tid; i < nk; i += blockDim.x) {
+            const int h = i / dk, j = i - h * dk;
+            kcache[(((size_t)pg * nkvh + h) * page_size + off) * dk + j] = from_f32<T>(row[nq + i]);
+        }
+    }
+    const float lam = (mix_mode == 2) ? lambda[0] : 0.f;
+    for (int i = tid; i < nv; i += blockDim.x) {
+        float v = row[nq + nk + i];
+        if (mix_mode == 1) v_keep[(size_t)t * nv + i] = v;
+        else if (mix_mode == 2) v = (1.0f - lam) * v + lam * v_keep[(size_t)t * nv + i];
+        if (slot >= 0 && vcache) {
+            const int h = i / dv, j = i - h * dv;
+            vcache[(((size_t)pg * nkvh + h) * page_size + off) * dv + j] = from_f32<T>(v);
+        }
+    }
+}
+
+IC_EXPORT int ic_qk_norm_store(const void* rows, int row_stride, int dtype, const float* bias, const float* qw,
+                               const float* kw, int norm_mode, float eps, int mix_mode, const float* lambda,
+                               float* v_keep, void* q_out, void* kcache, void* vcache, const int* slots, int T, int nh,
+                               int nkvh, int dk, int dv, int page_size, hipStream_t stream) {
+    if (T <= 0) return IC_OK;
+    if (nh <= 0 || nkvh <= 0 || dk <= 0 || dv <= 0 || page_size <= 0 || norm_mode < 0 || norm_mode > 2 || mix_mode < 0 ||
+        mix_mode > 2)
+        return IC_ERR_ARG;
+    if (nh + nkvh > 512) return IC_ERR_TOO_LARGE;
+    if (norm_mode != 0 && (qw == nullptr || kw == nullptr)) return IC_ERR_ARG;
+    if (mix_mode != 0 && v_keep == nullptr) return IC_ERR_ARG;
+    if (mix_mode == 2 && lambda == nullptr) return IC_ERR_ARG;
+    const long long n = (long long)(nh + nkvh) * dk + (long long)nkvh * dv;
+    if (row_stride < n) return IC_ERR_ARG;
+    const size_t lds = (size_t)n * sizeof(float);
+    if (lds > 60 * 1024) return IC_ERR_TOO_LARGE;
+    dim3 grid(T), block(256);
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, lds, stream, (const float*)rows, row_stride, bias, qw,
+                           kw, norm_mode, eps, mix_mode, lambda, v_keep, (float*)q_out, (float*)kcache, (float*)vcache,
+                           slots, nh, nkvh, dk, dv, page_size);
+    else if (dtype == IC_BF16)
+        hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, block, lds, stream, (const bf16*)rows, row_stride, bias, qw, kw,
+                           norm_mode, eps, mix_mode, lambda, v_keep, (bf16*)q_out, (bf16*)kcache, (bf16*)vcache, slots, nh,
+                           nkvh, dk, dv, page_size);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Element-wise activations of a dense feed-forward.  kind 0: relu(z)^2; 1: gelu_tanh(z); 2: silu(z).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float act_apply(float z, int kind) {
+    if (kind == 0) { const float r = fmaxf(z, 0.f); return r * r; }
+    if (kind == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return z / (1.0f + expf(-z));
+}
+
+template <typename T>
+__global__ void activation_kernel(const T* __restrict__ in, T* __restrict__ out, long long n, int kind) {
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        out[i] = from_f32<T>(act_apply(to_f32(in[i]), kind));
+}
+
+IC_EXPORT int ic_activation(const void* in, void* out, int dtype, long long n, int kind, hipStream_t stream) {
+    if (n <= 0) return IC_OK;
+    if (kind < 0 || kind > 2) return IC_ERR_ARG;
+    long long blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    dim3 grid((unsigned)blocks), block(256);
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(activation_kernel<float>, grid, block, 0, stream, (const float*)in, (float*)out, n, kind);
+    else if (dtype == IC_BF16)
+        hipLaunchKernelGGL(activation_kernel<bf16>, grid, block, 0, stream, (const bf16*)in, (bf16*)out, n, kind);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}

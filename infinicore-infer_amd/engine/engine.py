@@ -96,10 +96,11 @@ class Engine:
         keyed: Dict[tuple, List[int]] = {}
         for slot, need in enumerate(needs):
             if need.paged:
-                keyed.setdefault((need.planes, need.n_kv_heads, need.head_dim, need.window), []).append(slot)
+                keyed.setdefault((need.planes, need.n_kv_heads, need.head_dim, need.window, tuple(need.plane_dims),
+                                  need.keep_first if need.window else 0), []).append(slot)
         self.groups: List[GroupSpec] = [
-            GroupSpec("window" if w else "full", nkv, dh, w, tuple(slots), planes)
-            for (planes, nkv, dh, w), slots in keyed.items()]
+            GroupSpec("window" if w else "full", nkv, dh, w, tuple(slots), planes, dims, keep)
+            for (planes, nkv, dh, w, dims, keep), slots in keyed.items()]
         # positions a request may reach: the model's limit and that of every part (a table's length)
         limits = [model.spec.max_positions] + [p.position_limit() for p in model.all_parts()]
         self.max_positions = min(int(l) for l in limits if l is not None)
@@ -760,8 +761,8 @@ class _DecodeGraph:
                 if self._row_keys[g][r] != key:
                     base = o["tables%d" % g] + r * self.maxb
                     a[base:base + len(table)] = table
-                    if req.first_live[g]:
-                        a[base:base + req.first_live[g]] = 0     # pages given back are never read; keep the index valid
+                    if req.first_live[g]:                        # pages given back (-1) are never read; keep the index valid
+                        np.maximum(a[base:base + req.first_live[g]], 0, out=a[base:base + req.first_live[g]])
                     a[base + len(table):base + self.maxb] = 0
                     self._row_keys[g][r] = key
         self.ctx.host_state_slots = slots

@@ -51,6 +51,7 @@ def main(argv=None) -> int:
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
+    ap.add_argument("--max-requests", type=int, default=4, help="state slots: the most requests live at any time")
     ap.add_argument("--page-size", type=int, default=16, choices=(16, 32, 64))
     ap.add_argument("--device", default="cuda:0")
     ap.add_argument("--attention", default="auto", choices=("auto", "generic"))
@@ -59,7 +60,7 @@ def main(argv=None) -> int:
     print("[trace_run] loading kernels and model from %s (%s)" % (args.model, args.dtype),
           file=sys.stderr, flush=True)
     engine = Engine.from_dir(args.model, dtype=_DTYPES[args.dtype], device=args.device,
-                             max_tokens=args.max_tokens, page_size=args.page_size, max_requests=64,
+                             max_tokens=args.max_tokens, page_size=args.page_size, max_requests=args.max_requests,
                              attention_impl=args.attention)
     print("[trace_run] ready", file=sys.stderr, flush=True)
     replay(engine, sys.stdin, args.out)

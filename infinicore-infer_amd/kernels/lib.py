@@ -108,6 +108,11 @@ _SIGNATURES = {
     "ic_attn_prefill_parts_of_step": [_I, _I, _I, _I, _I, _I, _I, _c.POINTER(_I)],
     "ic_attn_prefill_split": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _LL, _P, _P],
     "ic_attn_prefill_counter_ints": [],
+    "ic_embed_sinusoid": [_P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _F, _P],
+    "ic_norm_into_stream": [_P, _I, _P, _P, _P, _P, _I, _I, _I, _F, _P],
+    "ic_qk_norm_store": [_P, _I, _I, _P, _P, _P, _I, _F, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "ic_activation": [_P, _P, _I, _LL, _I, _P],
+    "ic_attn_span_generic": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
     "ic_argmax_static_max_rows": [],

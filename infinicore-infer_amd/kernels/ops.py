@@ -649,3 +649,126 @@ def splitk_add_rmsnorm(parts, x, alpha: float, weight, out, eps: float):
     check(get_lib().ic_splitk_add_rmsnorm(parts.data_ptr(), S, M, x.data_ptr(), float(alpha), weight.data_ptr(), out.data_ptr(),
                                           d, float(eps), _stream()), "splitk_add_rmsnorm")
     return out
+
+
+# ---- decoders whose sublayers read the residual stream and are normalised on the way back -------------------------
+ACTIVATIONS = {"relu2": 0, "gelu_tanh": 1, "silu": 2}
+
+
+def embed_sinusoid(tokens, positions, table, freq, out, copy=None, scale: float = 1.0):
+    """out[t, 2i] = table[tokens[t], 2i] * scale + sin(positions[t] * freq[i]), out[t, 2i+1] = .. + cos(..);
+    out is float32 [T, d]; ``copy`` (optional, [T, d]) receives out rounded to its dtype."""
+    _dev(tokens, positions, table, freq, out, copy)
+    _i32(tokens, "tokens")
+    _i32(positions, "positions")
+    T, d = out.shape
+    _need(tokens.numel() == T and positions.numel() == T and table.dim() == 2 and table.shape[1] == d and d % 2 == 0,
+          "embed_sinusoid: shape mismatch")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous(), "embed_sinusoid: layout")
+    _need(freq.dtype == torch.float32 and freq.is_contiguous() and freq.numel() == d // 2, "embed_sinusoid: freq must be float32 [d/2]")
+    if copy is not None:
+        _need(tuple(copy.shape) == (T, d) and copy.is_contiguous(), "embed_sinusoid: copy layout")
+    check(get_lib().ic_embed_sinusoid(tokens.data_ptr(), positions.data_ptr(), table.data_ptr(), dtype_code(table.dtype),
+                                      freq.data_ptr(), out.data_ptr(), copy.data_ptr() if copy is not None else None,
+                                      dtype_code(copy.dtype) if copy is not None else 0, T, d, float(scale), _stream()),
+          "embed_sinusoid")
+    return out
+
+
+def norm_into_stream(y, weight, x, eps: float, bias=None, copy=None):
+    """x += rmsnorm(y + bias) * weight, row by row (x float32, in place); ``copy`` (optional) receives the new x
+    rounded to its dtype."""
+    _dev(y, weight, x, bias, copy)
+    T, d = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and tuple(y.shape) == (T, d),
+          "norm_into_stream: layout")
+    _need(weight.dtype == torch.float32 and weight.numel() == d and weight.is_contiguous(), "norm_into_stream: weight must be float32 [d]")
+    if bias is not None:
+        _need(bias.dtype == torch.float32 and bias.numel() == d and bias.is_contiguous(), "norm_into_stream: bias must be float32 [d]")
+    if copy is not None:
+        _need(tuple(copy.shape) == (T, d) and copy.is_contiguous(), "norm_into_stream: copy layout")
+    check(get_lib().ic_norm_into_stream(y.data_ptr(), dtype_code(y.dtype), bias.data_ptr() if bias is not None else None,
+                                        weight.data_ptr(), x.data_ptr(), copy.data_ptr() if copy is not None else None,
+                                        dtype_code(copy.dtype) if copy is not None else 0, T, d, float(eps), _stream()),
+          "norm_into_stream")
+    return x
+
+
+def qk_norm_store(rows, bias, q_weight, k_weight, norm_mode: int, eps: float, mix_mode: int, mix_lambda, v_keep, q_out,
+                  kcache, vcache, slots, n_heads: int, n_kv_heads: int, key_dim: int, value_dim: int, page_size: int):
+    """One pass over the projected rows [q | k | v | ..]: bias, query/key norm (0 none, 1 per head, 2 whole row), value
+    mixing (0 none, 1 keep the values in ``v_keep``, 2 mix with ``v_keep`` by ``mix_lambda``), q to ``q_out``, k and v
+    into the cache planes at ``slots`` (None: no cache write)."""
+    _dev(rows, bias, q_weight, k_weight, mix_lambda, v_keep, q_out, kcache, vcache, slots)
+    T = rows.shape[0]
+    nq, nk, nv = n_heads * key_dim, n_kv_heads * key_dim, n_kv_heads * value_dim
+    _need(rows.dim() == 2 and rows.stride(1) == 1 and rows.shape[1] >= nq + nk + nv, "qk_norm_store: rows too short")
+    _need(tuple(q_out.shape) == (T, nq) and q_out.is_contiguous() and q_out.dtype == rows.dtype, "qk_norm_store: q_out layout")
+    for v, n, what in ((bias, nq + nk + nv, "bias"), (q_weight, (key_dim, nq)[norm_mode == 2], "q weight"),
+                       (k_weight, (key_dim, nk)[norm_mode == 2], "k weight"), (mix_lambda, 1, "lambda")):
+        if v is not None:
+            _need(v.dtype == torch.float32 and v.is_contiguous() and v.numel() == n, "qk_norm_store: %s must be float32 [%d]" % (what, n))
+    _need(norm_mode == 0 or (q_weight is not None and k_weight is not None), "qk_norm_store: norm weights missing")
+    if mix_mode:
+        _need(v_keep is not None and v_keep.dtype == torch.float32 and v_keep.is_contiguous() and v_keep.numel() == T * nv,
+              "qk_norm_store: v_keep must be float32 [T, kv_heads * value_dim]")
+        _need(mix_mode == 1 or mix_lambda is not None, "qk_norm_store: lambda missing")
+    if slots is not None:
+        _i32(slots, "slots")
+        _need(slots.numel() == T, "qk_norm_store: slots/rows mismatch")
+        _need(kcache.dtype == rows.dtype and vcache.dtype == rows.dtype and kcache.is_contiguous() and vcache.is_contiguous()
+              and tuple(kcache.shape[1:]) == (n_kv_heads, page_size, key_dim)
+              and tuple(vcache.shape[1:]) == (n_kv_heads, page_size, value_dim) and kcache.shape[0] == vcache.shape[0],
+              "qk_norm_store: cache must be K [pages, kv_heads, page_size, key_dim], V [.., value_dim]")
+    p = lambda t: t.data_ptr() if t is not None else None
+    check(get_lib().ic_qk_norm_store(rows.data_ptr(), rows.stride(0), dtype_code(rows.dtype), p(bias), p(q_weight), p(k_weight),
+                                     int(norm_mode), float(eps), int(mix_mode), p(mix_lambda), p(v_keep), q_out.data_ptr(),
+                                     p(kcache) if slots is not None else None, p(vcache) if slots is not None else None,
+                                     p(slots), T, n_heads, n_kv_heads, key_dim, value_dim, page_size, _stream()),
+          "qk_norm_store")
+
+
+def activation(x, out, kind: str):
+    """out = act(x) element by element (relu2: relu(z)^2, gelu_tanh, silu)."""
+    _dev(x, out)
+    _need(x.is_contiguous() and out.is_contiguous() and x.shape == out.shape and x.dtype == out.dtype, "activation: layout")
+    _need(kind in ACTIVATIONS, "activation: kind %r (have %s)" % (kind, ", ".join(sorted(ACTIVATIONS))))
+    check(get_lib().ic_activation(x.data_ptr(), out.data_ptr(), dtype_code(x.dtype), x.numel(), ACTIVATIONS[kind], _stream()),
+          "activation")
+    return out
+
+
+def _span_common(q, out, gate, kcache, vcache, block_tables, n_heads, n_kv_heads, key_dim, value_dim, page_size):
+    _dev(q, out, gate, kcache, vcache, block_tables)
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * key_dim, "span attention: q layout")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_heads * value_dim and out.shape[0] == q.shape[0],
+          "span attention: out layout")
+    _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype, "span attention: dtypes differ")
+    if gate is not None:
+        _need(gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[1] >= n_heads * value_dim and gate.shape[0] == q.shape[0]
+              and gate.dtype == q.dtype, "span attention: gate layout")
+    _need(kcache.is_contiguous() and vcache.is_contiguous() and kcache.shape[0] == vcache.shape[0]
+          and tuple(kcache.shape[1:]) == (n_kv_heads, page_size, key_dim)
+          and tuple(vcache.shape[1:]) == (n_kv_heads, page_size, value_dim),
+          "span attention: cache must be K [pages, kv_heads, page_size, key_dim], V [.., value_dim]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+          "span attention: block_tables must be int32 [R, max_blocks]")
+    _need(n_heads % n_kv_heads == 0, "span attention: heads not a multiple of kv heads")
+
+
+def attention_span_generic(q, out, gate, kcache, vcache, block_tables, token_req, positions, n_heads, n_kv_heads, key_dim,
+                           value_dim, page_size, scale: float, window: int = 0, keep_first: int = 0, sink: bool = False):
+    """out[t, h] = sum_j p_j V_j over the keys j <= positions[t] with positions[t] - j < window or j < keep_first
+    (window 0: all), p = softmax of scale * q . K_j with ``sink`` added to the denominator; times sigmoid(gate)."""
+    _span_common(q, out, gate, kcache, vcache, block_tables, n_heads, n_kv_heads, key_dim, value_dim, page_size)
+    _i32(token_req, "token_req")
+    _i32(positions, "positions")
+    T = q.shape[0]
+    _need(token_req.numel() == T and positions.numel() == T, "span attention: T mismatch")
+    _need(key_dim <= 512 and value_dim <= 512, "span attention: head size above 512")
+    check(get_lib().ic_attn_span_generic(
+        q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), gate.data_ptr() if gate is not None else None,
+        gate.stride(0) if gate is not None else 0, dtype_code(q.dtype), kcache.data_ptr(), vcache.data_ptr(),
+        block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(), positions.data_ptr(), T, n_heads, n_kv_heads,
+        key_dim, value_dim, page_size, float(scale), int(window or 0), int(keep_first or 0), int(bool(sink)), _stream()),
+        "attention_span_generic")

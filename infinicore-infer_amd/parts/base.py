@@ -36,7 +36,10 @@ class CacheNeed:
     per token: planes = 1, n_kv_heads = 1, head_dim = its width), all tokens or a window of them;
     kind 'state': a fixed-size tensor of ``state_shape`` per request;
     kind 'kv+state': both, for a mixer that walks a paged cache and carries a running state as well;
-    kind 'none': nothing."""
+    kind 'none': nothing.
+    ``plane_dims``: the width of every plane when they differ (keys of 64 and values of 32 entries per head:
+    (64, 32)); empty: every plane is ``head_dim`` wide.  ``keep_first``: with a window, the first tokens of a
+    sequence that stay readable for good (their pages are never given back)."""
     kind: str = "none"
     n_kv_heads: int = 0
     head_dim: int = 0
@@ -44,6 +47,8 @@ class CacheNeed:
     state_shape: Tuple[int, ...] = ()
     state_dtype: torch.dtype = torch.float32
     planes: int = 2
+    plane_dims: Tuple[int, ...] = ()
+    keep_first: int = 0
 
     def __post_init__(self):
         if self.kind not in ("none", "kv", "state", "kv+state"):
@@ -53,6 +58,10 @@ class CacheNeed:
                              % (self.planes, self.n_kv_heads, self.head_dim))
         if self.has_state and not self.state_shape:
             raise ValueError("a state need names the state's shape")
+        if self.plane_dims and (len(self.plane_dims) != self.planes or min(self.plane_dims) <= 0):
+            raise ValueError("plane_dims names a positive width for each of the %d planes (got %r)" % (self.planes, self.plane_dims))
+        if self.keep_first < 0:
+            raise ValueError("keep_first must not be negative")
 
     @property
     def paged(self) -> bool:
@@ -94,6 +103,14 @@ class DeferredRows:
         T = self.values.shape[0]
         f = torch.rsqrt(self.sumsq.sum(0)[:T, None] / self.width + self.eps)
         return (self.values.to(torch.float32) * f).to(self.values.dtype)
+
+
+@dataclass
+class StreamCopy:
+    """Nothing is owed to the residual stream, and ``values`` hold it rounded to the compute dtype: what a block
+    whose sublayers read the stream itself hands to the next one (its last kernel wrote the copy along), so that
+    no cast kernel runs between layers.  Whoever cannot use it drops it."""
+    values: torch.Tensor
 
 
 @dataclass

@@ -10,7 +10,7 @@ it: the block leaves its last add pending for whoever normalises next.  For
 few rows the add and the norm go further, into the products on either side
 (``ResidualTail`` / ``DeferredRows``): then a layer is six kernels, not eight.
 """
-from .base import Block, DeferredRows, ResidualTail, register_part
+from .base import Block, DeferredRows, ResidualTail, StreamCopy, register_part
 
 
 @register_part("block", "prenorm_residual")
@@ -75,3 +75,52 @@ class PreNormResidualBlock(Block):
         if isinstance(y, DeferredRows):
             return y
         return (y, self.residual_scale)
+
+
+@register_part("block", "outnorm_residual")
+class OutputNormResidualBlock(Block):
+    """x += norm1(mixer(x)); x += norm2(ffn(x)): the sublayers read the residual stream itself and the norm sits on
+    their OUTPUT, on the way back into the stream (the second half only when the layer has a feed-forward).
+
+    The stream is float32; a sublayer's products want it in the compute dtype, so the kernel that updates the stream
+    (``forward_into_stream`` of the norm part) writes that copy along and the block hands it to the next one as
+    ``StreamCopy``: a layer is its products, the attention kernels and two row kernels.  A mixer that keeps its last
+    projection's bias back (``defers_bias``) has it added inside the norm kernel, before the sum of squares."""
+    graph_safe = True
+    accepts_stream_copy = True
+
+    def __init__(self, name, runtime, mixer=None, mixer_norm=None, feed_forward=None, feed_forward_norm=None):
+        super().__init__(name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm)
+        if mixer is None or mixer_norm is None:
+            raise ValueError("block %s: an output-norm residual block needs a mixer and its norm" % name)
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("block %s: a feed-forward and its norm come together, or neither" % name)
+        for n in (mixer_norm, feed_forward_norm):
+            if n is not None and not hasattr(n, "forward_into_stream"):
+                raise ValueError("block %s: norm part %s cannot normalise a sublayer's output into the stream"
+                                 % (name, type(n).__name__))
+
+    def _copy_buffer(self, x, ctx):
+        return None if self.runtime.dtype == x.dtype else ctx.ws.buffer("stream_copy", tuple(x.shape), self.runtime.dtype)
+
+    def forward(self, x, pending, ctx, cache):
+        if isinstance(pending, StreamCopy):
+            h = pending.values
+        else:
+            if pending is not None:
+                from ..kernels import ops
+                ops.residual_add(x, pending[0], pending[1])
+            h = self._copy_buffer(x, ctx)
+            h = x if h is None else h.copy_(x)
+        if getattr(self.mixer, "defers_bias", False):
+            y = self.mixer.forward(h, ctx, cache, defer_bias=True)
+            bias = self.mixer.deferred_bias()
+        else:
+            y, bias = self.mixer.forward(h, ctx, cache), None
+        copy = self._copy_buffer(x, ctx)
+        self.mixer_norm.forward_into_stream(y, x, copy=copy, bias=bias)
+        h = x if copy is None else copy
+        if self.feed_forward is not None:
+            y = self.feed_forward.forward(h, ctx)
+            self.feed_forward_norm.forward_into_stream(y, x, copy=copy)
+        return StreamCopy(h)

@@ -12,8 +12,15 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import WeightSpec
-from .base import DeferredRows, Part, register_part
+from .base import DeferredRows, Part, StreamCopy, register_part
 from .linear import linear
+
+
+def sinusoid_frequencies(width: int, base: float) -> torch.Tensor:
+    """f_i = base^(-2i/width) for i < width/2, in float32 arithmetic (the angle of position p is the float32
+    product p * f_i)."""
+    i = torch.arange(width // 2, dtype=torch.float32)
+    return torch.pow(torch.tensor(base, dtype=torch.float32), -2.0 * i / width).contiguous()
 
 
 @register_part("embedding", "embedding")
@@ -23,27 +30,43 @@ class Embedding(Part):
     category = "embedding"
 
     def __init__(self, name, runtime, vocab_size: int, hidden_size: int, scale: float = 1.0,
-                 fallback_name=None):
+                 fallback_name=None, tensor=None, sinusoid_base=None):
+        """``tensor``: the table's full name when it is not ``name + "weight"``.  ``sinusoid_base`` b: a position
+        vector is added to every row, entry 2i = sin(p b^(-2i/width)), entry 2i+1 = cos of the same angle."""
         super().__init__(name, runtime)
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.scale = float(scale)
         self.fallback = fallback_name + "weight" if fallback_name else None
+        self.tensor = tensor if tensor is not None else name + "weight"
         self.table = None
+        self.freq = None
+        if sinusoid_base is not None:
+            if hidden_size % 2:
+                raise ValueError("a sinusoidal position vector needs an even width (got %d)" % hidden_size)
+            self.freq = sinusoid_frequencies(hidden_size, float(sinusoid_base)).to(runtime.device)
+        self.takes_context = self.freq is not None      # forward wants the step's positions
 
     def weight_specs(self):
-        return {self.name + "weight": WeightSpec((self.vocab_size, self.hidden_size), "matrix", self.fallback)}
+        return {self.tensor: WeightSpec((self.vocab_size, self.hidden_size), "matrix", self.fallback)}
 
     def load_weights(self, tensors):
-        self.table = tensors[self.name + "weight"]
+        self.table = tensors[self.tensor]
 
-    def forward(self, tokens, x):
-        return ops.embed(tokens, self.table, x, self.scale)
+    def forward(self, tokens, x, ctx=None):
+        if self.freq is None:
+            return ops.embed(tokens, self.table, x, self.scale)
+        # the stream's copy in the compute dtype comes along (the first layer's sublayer may read the stream itself)
+        copy = None
+        if self.runtime.dtype != torch.float32:
+            copy = ctx.ws.buffer("stream_copy", tuple(x.shape), self.runtime.dtype)
+        ops.embed_sinusoid(tokens, ctx.positions, self.table, self.freq, x, copy=copy, scale=self.scale)
+        return StreamCopy(copy if copy is not None else x)
 
     def native_desc(self):
         """(table address, scale) for the native step function."""
         t = self.table
-        if not (self._forward_is(Embedding) and t is not None and t.is_cuda and t.dtype == self.runtime.dtype
-                and t.is_contiguous()):
+        if not (self._forward_is(Embedding) and self.freq is None and t is not None and t.is_cuda
+                and t.dtype == self.runtime.dtype and t.is_contiguous()):
             return None
         return (t.data_ptr(), self.scale)
 
@@ -66,21 +89,24 @@ class LMHead(Part):
     category = "head"
 
     def __init__(self, name, runtime, vocab_size: int, hidden_size: int, logit_scale: float = 1.0,
-                 fallback_name=None, tied: bool = False):
+                 fallback_name=None, tied: bool = False, tensor=None):
+        """``tensor``: the matrix's full name when it is not ``name + "weight"`` (the embedding's own tensor name: the
+        table is then held once and serves both)."""
         super().__init__(name, runtime)
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.logit_scale = float(logit_scale)
         self.fallback = fallback_name + "weight" if fallback_name else None
         self.tied = bool(tied) and self.fallback is not None
+        self.tensor = tensor if tensor is not None else name + "weight"
         self.weight = None
         self._scaled_norms = {}
 
     def weight_specs(self):
-        return {self.name + "weight": WeightSpec((self.vocab_size, self.hidden_size), "matrix", self.fallback,
-                                                 tied=self.tied)}
+        return {self.tensor: WeightSpec((self.vocab_size, self.hidden_size), "matrix", self.fallback,
+                                        tied=self.tied)}
 
     def load_weights(self, tensors):
-        self.weight = tensors[self.name + "weight"]
+        self.weight = tensors[self.tensor]
         self._scaled_norms = {}
 
     def deferred_norm(self, final_norm):

@@ -13,7 +13,7 @@ import torch
 from ..config.spec import ModelSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec, load_weights
-from .base import CacheNeed, DeferredRows, Runtime, build_part
+from .base import CacheNeed, DeferredRows, Runtime, StreamCopy, build_part
 
 
 class DecoderModel:
@@ -132,11 +132,16 @@ class DecoderModel:
         """Runs ctx.T tokens; returns float32 logits [len(ctx.want_rows), vocab] or None."""
         T = ctx.T
         x = ctx.ws.buffer("residual", (T, self.spec.hidden_size), torch.float32)
-        self.embedding.forward(ctx.tokens, x)
-        pending = None
+        if getattr(self.embedding, "takes_context", False):
+            pending = self.embedding.forward(ctx.tokens, x, ctx)      # may hand on the stream's copy (StreamCopy)
+        else:
+            self.embedding.forward(ctx.tokens, x)
+            pending = None
         last = len(self.schedule) - 1
         for i, e in enumerate(self.schedule):
             block = self.layers[e.layer]
+            if isinstance(pending, StreamCopy) and not getattr(block, "accepts_stream_copy", False):
+                pending = None                                        # nothing is owed; this block makes its own input
             if not block.fuses_successor:
                 if isinstance(pending, DeferredRows):
                     raise RuntimeError("block %s was handed half-normed rows it did not ask for" % block.name)
@@ -154,6 +159,8 @@ class DecoderModel:
             return None
         if isinstance(pending, DeferredRows):
             return self.head.forward(pending, ctx.want_rows, self.final_norm, ctx)
+        if isinstance(pending, StreamCopy):
+            pending = None
         if pending is not None:
             ops.residual_add(x, pending[0], pending[1])
         return self.head.forward(x, ctx.want_rows, self.final_norm, ctx)

@@ -13,17 +13,27 @@ from .base import Norm, register_part
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, name, runtime, size: int, eps: float):
+    def __init__(self, name, runtime, size: int, eps: float, weight_offset: float = 0.0, tensor=None):
+        """``weight_offset``: what is added to the stored weight (1.0 for weights stored around zero, y = x r (1 + w));
+        the sum is formed once, in float32, when the weights are loaded.  ``tensor``: the weight's full name when it
+        is not ``name + "weight"``."""
         super().__init__(name, runtime)
         self.size = size
         self.eps = float(eps)
+        self.weight_offset = float(weight_offset)
+        self.tensor = tensor if tensor is not None else name + "weight"
         self.weight = None
 
     def weight_specs(self):
-        return {self.name + "weight": WeightSpec((self.size,), "vector")}
+        return {self.tensor: WeightSpec((self.size,), "vector")}
 
     def load_weights(self, tensors):
-        self.weight = tensors[self.name + "weight"]
+        w = tensors[self.tensor]
+        self.weight = (w.to(torch.float32) + self.weight_offset).contiguous() if self.weight_offset else w
+
+    def forward_into_stream(self, y, x, copy=None, bias=None):
+        """x += norm(y + bias), the norm on a sublayer's output; ``copy`` receives the new x in its dtype."""
+        return ops.norm_into_stream(y, self.weight, x, self.eps, bias=bias, copy=copy)
 
     def forward(self, x, out, rows=None, out_scale: float = 1.0):
         return ops.rmsnorm(x, self.weight, out, self.eps, out_scale, rows)

@@ -65,12 +65,14 @@ class WeightSpec:
     hold both they must be equal, and one copy is kept.  ``pack`` = (name, place):
     tensors with the same pack name are laid out one after the other in the order
     of ``place``, and the loader also hands out their concatenation along the rows
-    under that name without copying (fused projections)."""
+    under that name without copying (fused projections).  ``optional``: the files may lack the
+    tensor (it is then absent from the result); when they hold it, it is checked and loaded."""
     shape: Tuple[int, ...]
     role: str = "matrix"
     fallback: Optional[str] = None
     tied: bool = False
     pack: Optional[Tuple[str, int]] = None
+    optional: bool = False
 
 
 # Non-parameter buffers that some exporters write; never needed, never an error.
@@ -181,6 +183,8 @@ def load_weights(model_dir: str, specs: Dict[str, WeightSpec], compute_dtype: to
     tied_pairs = []
     for name, spec in specs.items():
         src = name if name in where else (spec.fallback if spec.fallback in where else None)
+        if src is None and spec.optional:
+            continue
         if src is None:
             missing.append(name if not spec.fallback else "%s (or %s)" % (name, spec.fallback))
             continue
@@ -272,7 +276,7 @@ def load_weights(model_dir: str, specs: Dict[str, WeightSpec], compute_dtype: to
         key = (src, dt)
         if key not in views:                 # two names of one stored tensor get the same tensor object
             o = place[key]
-            views[key] = arena[o:o + _nbytes(specs[name].shape, dt)].view(dt).view(*specs[name].shape)
+            views[key] = arena[o:o + _nbytes(specs[name].shape, dt)].view(dt).view(tuple(specs[name].shape))
         out[name] = views[key]
     for pname, (o, dt, shape) in packed_ok.items():
         out[pname] = arena[o:o + _nbytes(shape, dt)].view(dt).view(*shape)
