@@ -82,6 +82,15 @@ int ic_activation(const void* in, void* out, int dtype, long long n, int kind, h
 // softmax's denominator; gate (nullable): out *= sigmoid(gate[t, h dv + d]).
 int ic_attn_span_generic(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* token_req, const int* positions, int T, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, hipStream_t stream);
 
+// Single new tokens, split over the visible keys (key and value sizes 32, 64, 128; float32 or bfloat16).  tok_list (nullable): the rows that are
+// single tokens.  part_acc: float32 [n_tok, nh, nsplit, dv]; part_ml: float32 [n_tok, nh, nsplit, 2]; nsplit <= 32 (1: no second pass, no scratch).
+int ic_attn_span_decode_supported(int dtype, int dk, int dv);
+int ic_attn_span_decode_splits(int n_rows, int n_kv_heads, int max_keys, int compute_units);
+int ic_attn_span_decode(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tok_list, const int* token_req, const int* positions, float* part_acc, float* part_ml, int n_tok, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, int nsplit, hipStream_t stream);
+// Prompt portions on the matrix cores (bfloat16; key and value sizes 32, 64, 128; scale > 0).  tiles as for ic_attn_prefill, rows <= 128.
+int ic_attn_span_prefill_supported(int dtype, int dk, int dv);
+int ic_attn_span_prefill(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dk, int dv, int page_size, float scale, int window, int keep_first, int sink, hipStream_t stream);
+
 // ---- gemm.hip ---------------------------------------------------------------------------------------
 // A norm y = x * rsqrt(mean(x^2) + eps) * w between two products of M <= 16 rows can be split over them: the
 // product before it adds its result to the residual stream, stores x * w and the sums of x^2 per row and

@@ -113,6 +113,11 @@ _SIGNATURES = {
     "ic_qk_norm_store": [_P, _I, _I, _P, _P, _P, _I, _F, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "ic_activation": [_P, _P, _I, _LL, _I, _P],
     "ic_attn_span_generic": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "ic_attn_span_decode_supported": [_I, _I, _I],
+    "ic_attn_span_decode_splits": [_I, _I, _I, _I],
+    "ic_attn_span_decode": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
+    "ic_attn_span_prefill_supported": [_I, _I, _I],
+    "ic_attn_span_prefill": [_P, _I, _P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
     "ic_argmax_static_max_rows": [],

@@ -772,3 +772,61 @@ def attention_span_generic(q, out, gate, kcache, vcache, block_tables, token_req
         block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(), positions.data_ptr(), T, n_heads, n_kv_heads,
         key_dim, value_dim, page_size, float(scale), int(window or 0), int(keep_first or 0), int(bool(sink)), _stream()),
         "attention_span_generic")
+
+
+def attention_span_decode_supported(dtype, key_dim: int, value_dim: int) -> bool:
+    code = _code_or_none(dtype)
+    return code is not None and bool(get_lib().ic_attn_span_decode_supported(code, key_dim, value_dim))
+
+
+def attention_span_decode_splits(n_rows: int, n_kv_heads: int, max_keys: int, compute_units: int) -> int:
+    return int(get_lib().ic_attn_span_decode_splits(n_rows, n_kv_heads, max_keys, compute_units))
+
+
+def attention_span_decode(q, out, gate, kcache, vcache, block_tables, tok_list, n_tok, token_req, positions, part_acc,
+                          part_ml, n_heads, n_kv_heads, key_dim, value_dim, page_size, scale: float, window: int = 0,
+                          keep_first: int = 0, sink: bool = False, n_split: int = 1):
+    """The rows ``tok_list`` (None: rows 0..n_tok-1) of q, each a request's single new token, split ``n_split`` ways
+    over their visible keys.  part_acc / part_ml: float32 scratch of n_tok * heads * n_split * (value_dim / 2) elements."""
+    _span_common(q, out, gate, kcache, vcache, block_tables, n_heads, n_kv_heads, key_dim, value_dim, page_size)
+    _i32(token_req, "token_req")
+    _i32(positions, "positions")
+    if tok_list is not None:
+        _i32(tok_list, "tok_list")
+        _need(tok_list.numel() >= n_tok, "span decode: tok_list shorter than n_tok")
+    else:
+        _need(n_tok <= q.shape[0], "span decode: more tokens than rows")
+    _need(1 <= n_split <= 32, "span decode: 1..32 splits")
+    if n_split > 1:
+        _dev(part_acc, part_ml)
+        _need(part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32
+              and part_acc.numel() >= n_tok * n_heads * n_split * value_dim
+              and part_ml.numel() >= n_tok * n_heads * n_split * 2, "span decode: scratch too small")
+    check(get_lib().ic_attn_span_decode(
+        q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), gate.data_ptr() if gate is not None else None,
+        gate.stride(0) if gate is not None else 0, dtype_code(q.dtype), kcache.data_ptr(), vcache.data_ptr(),
+        block_tables.data_ptr(), block_tables.stride(0), tok_list.data_ptr() if tok_list is not None else None,
+        token_req.data_ptr(), positions.data_ptr(), part_acc.data_ptr() if n_split > 1 else None,
+        part_ml.data_ptr() if n_split > 1 else None, n_tok, n_heads, n_kv_heads, key_dim, value_dim, page_size,
+        float(scale), int(window or 0), int(keep_first or 0), int(bool(sink)), int(n_split), _stream()),
+        "attention_span_decode")
+
+
+def attention_span_prefill_supported(dtype, key_dim: int, value_dim: int) -> bool:
+    code = _code_or_none(dtype)
+    return code is not None and bool(get_lib().ic_attn_span_prefill_supported(code, key_dim, value_dim))
+
+
+def attention_span_prefill(q, out, gate, kcache, vcache, block_tables, tiles, n_tiles, n_heads, n_kv_heads, key_dim,
+                           value_dim, page_size, scale: float, window: int = 0, keep_first: int = 0, sink: bool = False):
+    """Prompt portions listed as tiles int32 [n_tiles, 4] (request row, first token row, rows, first position)."""
+    _span_common(q, out, gate, kcache, vcache, block_tables, n_heads, n_kv_heads, key_dim, value_dim, page_size)
+    _dev(tiles)
+    _need(tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.numel() >= 4 * n_tiles, "span prefill: tiles layout")
+    _need(scale > 0, "span prefill: the scale must be positive")
+    check(get_lib().ic_attn_span_prefill(
+        q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), gate.data_ptr() if gate is not None else None,
+        gate.stride(0) if gate is not None else 0, dtype_code(q.dtype), kcache.data_ptr(), vcache.data_ptr(),
+        block_tables.data_ptr(), block_tables.stride(0), tiles.data_ptr(), n_tiles, n_heads, n_kv_heads, key_dim, value_dim,
+        page_size, float(scale), int(window or 0), int(keep_first or 0), int(bool(sink)), _stream()),
+        "attention_span_prefill")

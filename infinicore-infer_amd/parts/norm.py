@@ -25,7 +25,7 @@ class RMSNorm(Norm):
         self.weight = None
 
     def weight_specs(self):
-        return {self.tensor: WeightSpec((self.size,), "vector")}
+        return {self.tensor: WeightSpec((self.size,), "vector", mean=(1.0 - self.weight_offset) if self.weight_offset else None)}
 
     def load_weights(self, tensors):
         w = tensors[self.tensor]

@@ -82,18 +82,18 @@ class SpanAttention(Mixer):
         if self.gate:
             specs[n + "g"] = WeightSpec((self.na, d), pack=(pack, 3))
         if self.qkv_bias:
-            specs[n + "q.b"] = WeightSpec((self.nq,), "vector", pack=(bpack, 0))
-            specs[n + "k.b"] = WeightSpec((self.nk,), "vector", pack=(bpack, 1))
-            specs[n + "v.b"] = WeightSpec((self.nv,), "vector", pack=(bpack, 2))
+            specs[n + "q.b"] = WeightSpec((self.nq,), "vector", pack=(bpack, 0), mean=0.0)
+            specs[n + "k.b"] = WeightSpec((self.nk,), "vector", pack=(bpack, 1), mean=0.0)
+            specs[n + "v.b"] = WeightSpec((self.nv,), "vector", pack=(bpack, 2), mean=0.0)
         if self.out_bias:
-            specs[n + "o.b"] = WeightSpec((d,), "vector")
+            specs[n + "o.b"] = WeightSpec((d,), "vector", mean=0.0)
         if self.norm_mode:
             per_head = self.norm_mode == 1
             specs[n + "q.norm"] = WeightSpec((self.dk if per_head else self.nq,), "vector")
             specs[n + "k.norm"] = WeightSpec((self.dk if per_head else self.nk,), "vector")
         if self.mix_mode or self.mix_optional:
             # the keeping layer holds a scalar too, which nothing reads
-            specs[n + "vmix"] = WeightSpec((), "vector", optional=self.mix_mode == 0)
+            specs[n + "vmix"] = WeightSpec((), "vector", optional=self.mix_mode == 0, mean=0.5)
         return specs
 
     def load_weights(self, tensors):
@@ -142,6 +142,35 @@ class SpanAttention(Mixer):
         return y
 
     def _attend(self, q, out, gate, ctx, cache):
-        ops.attention_span_generic(q, out, gate, cache.k, cache.v, cache.block_tables, ctx.token_req, ctx.positions,
-                                   self.nh, self.nkvh, self.dk, self.dv, ctx.page_size, self.scale, self.window,
-                                   self.keep_first, self.sink)
+        """Single-token rows go to the split-key kernel, prompt portions to the matrix-core kernel, where the sizes
+        have one (and the runtime does not ask for the general kernel alone); everything else to the general kernel."""
+        rt = self.runtime
+        args = (self.nh, self.nkvh, self.dk, self.dv, ctx.page_size, self.scale, self.window, self.keep_first, self.sink)
+        n_dec, n_tiles = ctx.n_decode_rows, ctx.n_prefill_tiles
+        tiled = rt.attention_impl == "auto" and n_dec + n_tiles > 0
+        use_dec = tiled and n_dec > 0 and ops.attention_span_decode_supported(rt.dtype, self.dk, self.dv)
+        use_pre = tiled and n_tiles > 0 and self.scale > 0 and ops.attention_span_prefill_supported(rt.dtype, self.dk, self.dv)
+        if not (use_dec or n_dec == 0) or not (use_pre or n_tiles == 0) or not tiled:
+            ops.attention_span_generic(q, out, gate, cache.k, cache.v, cache.block_tables, ctx.token_req, ctx.positions, *args)
+            return
+        if use_dec:
+            n_split = self._key_splits(ctx)
+            part_acc = part_ml = None
+            if n_split > 1:
+                part_acc = ctx.ws.buffer("span_part_acc", (n_dec * self.nh * n_split * self.dv,), torch.float32)
+                part_ml = ctx.ws.buffer("span_part_ml", (n_dec * self.nh * n_split * 2,), torch.float32)
+            ops.attention_span_decode(q, out, gate, cache.k, cache.v, cache.block_tables,
+                                      None if ctx.decode_rows_identity else ctx.decode_rows, n_dec, ctx.token_req,
+                                      ctx.positions, part_acc, part_ml, *args, n_split=n_split)
+        if use_pre:
+            ops.attention_span_prefill(q, out, gate, cache.k, cache.v, cache.block_tables, ctx.prefill_tiles, n_tiles, *args)
+
+    def _key_splits(self, ctx) -> int:
+        """Ways to split the visible keys of single-token rows: the kernel library's rule, from the number of rows and
+        the most keys a row can see (the step's rounded key count, or the window with its kept keys when smaller)."""
+        if ctx.fixed_decode_splits is not None:
+            return max(1, min(32, ctx.fixed_decode_splits))
+        most = ctx.max_context or 1
+        if self.window:
+            most = min(most, self.window + self.keep_first)
+        return ops.attention_span_decode_splits(ctx.n_decode_rows, self.nkvh, most, ctx.cu_count)

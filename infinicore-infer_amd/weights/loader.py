@@ -66,13 +66,16 @@ class WeightSpec:
     tensors with the same pack name are laid out one after the other in the order
     of ``place``, and the loader also hands out their concatenation along the rows
     under that name without copying (fused projections).  ``optional``: the files may lack the
-    tensor (it is then absent from the result); when they hold it, it is checked and loaded."""
+    tensor (it is then absent from the result); when they hold it, it is checked and loaded.
+    ``mean``: the value a vector is drawn around in random-weights mode (default 1: a scale; 0 for a bias
+    or a weight stored around zero)."""
     shape: Tuple[int, ...]
     role: str = "matrix"
     fallback: Optional[str] = None
     tied: bool = False
     pack: Optional[Tuple[str, int]] = None
     optional: bool = False
+    mean: Optional[float] = None
 
 
 # Non-parameter buffers that some exporters write; never needed, never an error.

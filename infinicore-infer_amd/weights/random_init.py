@@ -7,7 +7,8 @@ neither on the order in which tensors are drawn, nor on the device that draws
 them, nor on how a tensor is cut into pieces while it is drawn.  So a folder
 written on the CPU and weights drawn straight into a model on the GPU are the
 same model.  Matrices and tables are N(0, std) in float32, rounded to the storage
-dtype; norm weights are 1, or N(1, norm_std).
+dtype; vectors are their spec's mean (1 for a scale, 0 for a bias or a weight stored
+around zero), or N(mean, norm_std).
 
 The draw uses integer arithmetic and one multiplication only, which give the same
 bits everywhere: two 64-bit words per element from a counter hash (splitmix64's
@@ -76,12 +77,12 @@ def standard_normal(seed: int, name: str, n: int, device="cpu") -> torch.Tensor:
     return out
 
 
-def _draw(seed: int, name: str, shape, role: str, std: float, norm_std: float, device) -> torch.Tensor:
+def _draw(seed: int, name: str, shape, role: str, std: float, norm_std: float, device, mean=None) -> torch.Tensor:
     n = 1
     for d in shape:
         n *= int(d)
     if role == "vector":
-        t = torch.ones(shape, dtype=torch.float32, device=device)
+        t = torch.full(tuple(shape), 1.0 if mean is None else float(mean), dtype=torch.float32, device=device)
         if norm_std:
             t = t + norm_std * standard_normal(seed, name, n, device).view(shape)
         return t
@@ -104,7 +105,7 @@ def random_state_dict(config: dict, seed: int, std: float = 0.02, norm_std: floa
     for name, spec in specs.items():
         if tie and spec.fallback in specs and spec.fallback in out:
             continue                # a tied tensor is not written: the loader takes the tensor it falls back to
-        t = _draw(seed, name, spec.shape, spec.role, std, norm_std, device)
+        t = _draw(seed, name, spec.shape, spec.role, std, norm_std, device, spec.mean)
         out[name] = (t if spec.role == "vector" else t.to(dtype)).contiguous()
     return out
 
@@ -120,7 +121,7 @@ def init_random_weights(model, seed: int, std: float = 0.02, norm_std: float = 0
         if tie and spec.fallback in specs and spec.fallback in tensors:
             tensors[name] = tensors[spec.fallback]
             continue
-        t = _draw(seed, name, spec.shape, spec.role, std, norm_std, rt.device)
+        t = _draw(seed, name, spec.shape, spec.role, std, norm_std, rt.device, spec.mean)
         tensors[name] = t if spec.role == "vector" else t.to(rt.dtype)
     model.load_weights(tensors)
 
