@@ -12,6 +12,9 @@ seeded uniform-random token ids.  One JSON line is printed.
   --workload mixed   the 1B shape's workload: 64 requests, prompts of 128..2,048 tokens, portions of 512
   --workload long    the 8B shape's workload: 4 prompts of 16,384 tokens, then decoding
   --direct           decode by calling the step function directly, without the scheduler
+  --workload designs the Fopezen decoder beside the MiniCPM decoder at equal layer sizes (a few layers of three real
+                     models' sizes): prefill and decode throughput of both, with the fraction of the memory or
+                     matrix-core peak each reaches (--only fopezen|minicpm: one of them, for a profiler)
 """
 import argparse
 import json
@@ -176,6 +179,96 @@ def time_decode(engine, batch, steps, warmup, vocab, seed=0):
     return dt / steps, (ctx0 + ctx1) / 2.0
 
 
+# Layer sizes for --workload designs: (width, heads, kv heads, head size, feed-forward, vocabulary).  The Fopezen model has the
+# same width, heads, kv heads and key size; its value size, window and kept keys are listed beside.
+DESIGN_SIZES = {
+    "2b-like": dict(width=2304, heads=36, kv=36, dim=64, ff=5760, vocab=32000, vdim=64, window=1024, keep=4),
+    "8b-like": dict(width=4096, heads=32, kv=8, dim=128, ff=14336, vocab=32000, vdim=128, window=2048, keep=16),
+    "1b-like": dict(width=1536, heads=24, kv=8, dim=64, ff=3840, vocab=32000, vdim=32, window=512, keep=4),
+}
+
+
+def _design_configs(z, layers):
+    mini = dict(model_type="minicpm", vocab_size=z["vocab"], hidden_size=z["width"], num_hidden_layers=layers,
+                num_attention_heads=z["heads"], num_key_value_heads=z["kv"], head_dim=z["dim"], intermediate_size=z["ff"],
+                max_position_embeddings=8192, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True, eos_token_id=[])
+    mixer = lambda w, k: dict(heads=z["heads"], kv_heads=z["kv"], dim=z["dim"], vdim=z["vdim"], scale=z["dim"] ** -0.5,
+                              mask=dict(size=w, keep_first=k), v_mix=True)
+    kinds = ["attention", "attention", "attention_2", "attention"]
+    fop = dict(architecture="Fopezen", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-5),
+               layers=[dict(type=kinds[i % 4], mixer=mixer(z["window"], z["keep"]), mlp=dict(kind="dense", ff=z["ff"]))
+                       for i in range(layers)])
+    return {"minicpm": mini, "fopezen": fop}
+
+
+def _design_numbers(design, z, layers, kinds=None):
+    """(weight bytes a decode step reads, cache bytes a decode step reads per request at context n, prefill flops at T)."""
+    d, H, G, dk, ff, V = z["width"], z["heads"], z["kv"], z["dim"], z["ff"], z["vocab"]
+    eb = _elem_bytes()
+    if design == "minicpm":
+        per_layer = (H + 2 * G) * dk * d + H * dk * d + 3 * d * ff
+        kv = lambda n: 2 * layers * G * dk * eb * n
+        attn = lambda T: layers * H * dk * 4.0 * (T * (T + 1) / 2)
+    else:
+        dv, w, keep = z["vdim"], z["window"], z["keep"]
+        gated = sum(1 for i in range(layers) if i % 4 != 2)
+        per_layer = (H * dk + G * dk + G * dv) * d + H * dv * d + 2 * d * ff
+        per_layer += gated / layers * H * dv * d
+        seen = lambda n: min(n, w + keep)
+        kv = lambda n: layers * G * (dk + dv) * eb * seen(n)
+        attn = lambda T: layers * H * (dk + dv) * 2.0 * sum(seen(i + 1) for i in range(T))
+    weights = eb * (layers * per_layer + V * d)
+    return weights, kv, (lambda T: 2.0 * T * layers * per_layer + attn(T) + 2.0 * V * d)
+
+
+def run_designs(args):
+    """Prefill and decode of the two decoders at equal layer sizes.  Decoding calls the step function directly (recorded
+    steps), greedy sampling on the device; a row gives tokens/s and what fraction of the memory bandwidth (decoding:
+    weights once + the cache rows a step reads) or of the matrix-core peak (prefill) that is."""
+    global PROMPT
+    from infinicore_infer_amd.config import config_from_dict
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.parts import Runtime, build_model
+    from infinicore_infer_amd.weights import init_random_weights
+    PROMPT = args.prompt
+    layers = args.layers or 4
+    dname = "bf16" if DTYPE == torch.bfloat16 else "fp32"
+    batches = [args.batch] if args.no_points else [1, 8, 64]
+    rows = []
+    for size in (args.sizes.split(",") if args.sizes else list(DESIGN_SIZES)):
+        z = DESIGN_SIZES[size]
+        for design, cfg in _design_configs(z, layers).items():
+            if args.only and design != args.only:
+                continue
+            conf = config_from_dict(cfg)
+            model = build_model(conf.model_spec(), Runtime(dtype=DTYPE, device="cuda:0"))
+            init_random_weights(model, seed=0, std=0.02, norm_std=0.02)
+            per_req = (PROMPT + args.warmup + args.steps + 128 + 63) // 64 * 64
+            engine = Engine(model, max_tokens=per_req * max(batches), page_size=args.page_size, max_requests=max(batches) + 1)
+            if args.eager:
+                engine.use_graphs = False
+            if not args.no_tune:
+                engine.tune_library_products([PROMPT] + [b for b in batches if b > 16])
+            weights, kv, pf_flops = _design_numbers(design, z, layers)
+            g = torch.Generator().manual_seed(5)
+            t_pf = time_prefill(engine, torch.randint(0, z["vocab"], (PROMPT,), generator=g).tolist(), reps=4)
+            row = {"size": size, "design": design, "layers": layers,
+                   "prefill_tokens_per_s": round(PROMPT / t_pf, 1), "prefill_ms": round(t_pf * 1e3, 3),
+                   "prefill_frac_of_matrix_peak": round(pf_flops(PROMPT) / t_pf / (PEAK_TFLOPS[dname] * 1e12), 4), "decode": {}}
+            for b in batches:
+                dt, ctx = time_decode(engine, b, args.steps, args.warmup, z["vocab"], seed=b)
+                row["decode"]["batch %d" % b] = {"tokens_per_s": round(b / dt, 1), "ms_per_step": round(dt * 1e3, 4),
+                                                 "frac_of_hbm_peak": round((weights + b * kv(ctx)) / dt / 1e9 / HBM_PEAK_GBS, 4)}
+            rows.append(row)
+            print(json.dumps(row), file=sys.stderr, flush=True)
+            del engine, model
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "prefill and decode tokens/s of two decoder designs at equal layer sizes", "unit": "tokens/s",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": dname, "prompt": PROMPT,
+                      "data": "synthetic (seeded random weights and token ids)", "rows": rows}))
+    return 0
+
+
 def run_mixed(args):
     """The 1B-shaped configuration's workload: 64 requests with prompts of 128..2,048 tokens go through the
     scheduler, which cuts the prompts into portions of 512 under a token budget per step and decodes the
@@ -262,7 +355,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES), help="2b is the benchmark's configuration (default; 1b for --workload mixed)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long"],
+    ap.add_argument("--sizes", default=None, help="--workload designs: comma-separated sizes (default: all of 2b-like, 8b-like, 1b-like)")
+    ap.add_argument("--only", default=None, choices=["fopezen", "minicpm"], help="--workload designs: one design only")
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long", "designs"],
                     help="decode: the benchmark (prefill of one prompt, decode steps at fixed batches); "
                          "mixed: 64 requests of 128..2048 prompt tokens through the scheduler, --steps tokens generated each; "
                          "long: the 8B shape with 4 prompts of 16,384 tokens (the same as --shape 8b --prompt 16384 --batch 4 --no-points)")
@@ -285,6 +380,10 @@ def main():
         return 2
 
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    if args.workload == "designs":
+        if args.steps == ap.get_default("steps"):
+            args.steps = 64
+        return run_designs(args)
     if args.workload == "long":
         args.shape = args.shape or "8b"
         if args.prompt == ap.get_default("prompt"):

@@ -229,16 +229,27 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
 #pragma unroll
             for (int i = 0; i < NVS * VEC; ++i) acc[j][i] = 0.f;
         }
-        for (int ib = lo + wave * KPW + grp; ib - grp - wave * KPW < hi; ib += kSdUnroll * KPW * kSdWaves) {
+        // The page ids of an iteration's keys are looked up one iteration ahead: an iteration then waits for one trip to
+        // memory (its rows), not for two in a row (page id, then row).
+        constexpr int STEP = kSdUnroll * KPW * kSdWaves;
+        int keyn[kSdUnroll], pgn[kSdUnroll];
+        auto look = [&](int ib) {
+#pragma unroll
+            for (int u = 0; u < kSdUnroll; ++u) {
+                const int idx = ib + u * KPW * kSdWaves;
+                keyn[u] = span_key(runs, idx < hi ? idx : hi - 1);         // a stand-in key that is a real one
+                pgn[u] = bt[keyn[u] / page_size];
+            }
+        };
+        const int ib0 = lo + wave * KPW + grp;
+        if (lo < hi) look(ib0);
+        for (int ib = ib0; ib - grp - wave * KPW < hi; ib += STEP) {
             float kf[kSdUnroll][VEC], vf[kSdUnroll][NVS * VEC];
             bool ok[kSdUnroll];
 #pragma unroll
             for (int u = 0; u < kSdUnroll; ++u) {
-                const int idx = ib + u * KPW * kSdWaves;
-                ok[u] = idx < hi;
-                const int key = span_key(runs, ok[u] ? idx : hi - 1);      // a stand-in key that is a real one
-                const int lp = key / page_size;
-                const size_t rowi = ((size_t)bt[lp] * nkvh + kvh) * page_size + (key - lp * page_size);
+                ok[u] = ib + u * KPW * kSdWaves < hi;
+                const size_t rowi = ((size_t)pgn[u] * nkvh + kvh) * page_size + (keyn[u] % page_size);
                 SpanVec<T>::load(kcache + rowi * DK + sub * VEC, kf[u]);
 #pragma unroll
                 for (int s = 0; s < NVS; ++s) {
@@ -248,6 +259,7 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
                         for (int i = 0; i < VEC; ++i) vf[u][s * VEC + i] = 0.f;
                 }
             }
+            if (ib + STEP - grp - wave * KPW < hi) look(ib + STEP);
 #pragma unroll
             for (int j = 0; j < kSdGQ; ++j) {
                 float s[kSdUnroll];
@@ -462,15 +474,10 @@ typedef __bf16 sp_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float sp_v16f __attribute__((ext_vector_type(16)));
 typedef float sp_v8f __attribute__((ext_vector_type(8)));
 typedef short sp_v4s __attribute__((ext_vector_type(4)));
+typedef unsigned sp_v4u __attribute__((ext_vector_type(4)));
 
 constexpr int kSpRows = 128;      // query rows per block
 constexpr int kSpKeys = 64;       // keys per step
-
-union SpFrag {
-    uint4 u;
-    uint2 h[2];
-    sp_bf16x8 v;
-};
 
 template <int DK, int DV>
 __global__ void __launch_bounds__(256, 2)
@@ -478,7 +485,7 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                          const uint16_t* __restrict__ gate, int gate_stride,
                          const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                          const int* __restrict__ block_tables, int bt_stride, const int4* __restrict__ tiles,
-                         int nh, int nkvh, int page_size, float scale_log2e, int window, int keep_first, int sink) {
+                         int nh, int nkvh, int page_shift, float scale_log2e, int window, int keep_first, int sink) {
     constexpr int NC = DK / 16;           // 16-wide chunks of the key size
     constexpr int ND = DV / 32;           // 32-row tiles of O^T
     constexpr int PK = DK + 8;            // padded row pitches in LDS (elements)
@@ -487,8 +494,11 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     constexpr int NLK = kSpKeys * KCH / 256, NLV = kSpKeys * VCH / 256;     // loads per thread and step
     static_assert(DK % 32 == 0 && DV % 32 == 0, "a step's rows split evenly over the block");
 
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[kSpKeys * PK];
-    __shared__ __attribute__((aligned(16))) uint16_t Vs[kSpKeys * PV];
+    // two stages: a step is computed from one while the next step's rows are written into the other (one barrier a step)
+    __shared__ __attribute__((aligned(16))) uint16_t Ks0[kSpKeys * PK];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs0[kSpKeys * PV];
+    __shared__ __attribute__((aligned(16))) uint16_t Ks1[kSpKeys * PK];
+    __shared__ __attribute__((aligned(16))) uint16_t Vs1[kSpKeys * PV];
 
     const int slot = (int)blockIdx.x;
     const int h = slot % nh;
@@ -498,6 +508,7 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     const int* bt = block_tables + (size_t)req * bt_stride;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int lq = lane & 31, half = lane >> 5;
+    const int page_size = 1 << page_shift, page_mask = page_size - 1;      // pages are a power of two here
 
     const int my_row = 32 * wave + lq;
     const bool row_ok = my_row < n_rows;
@@ -519,14 +530,11 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
         else { kb = win_kb0 + (s - kept_steps) * kSpKeys; klo = first_key; khi = last_key; }
     };
 
-    SpFrag qf[NC];
+    sp_bf16x8 qf[NC];
     {
-        const uint16_t* qp = q + (size_t)(row0 + my_row) * q_stride + (size_t)h * DK + 8 * half;
+        const uint16_t* qp = q + (size_t)(row0 + (row_ok ? my_row : 0)) * q_stride + (size_t)h * DK + 8 * half;
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            if (row_ok) qf[c].u = *reinterpret_cast<const uint4*>(qp + 16 * c);
-            else qf[c].u = make_uint4(0, 0, 0, 0);
-        }
+        for (int c = 0; c < NC; ++c) qf[c] = *reinterpret_cast<const sp_bf16x8*>(qp + 16 * c);      // rows beyond the tile read row 0 and are never written
     }
     sp_v16f oacc[ND];
 #pragma unroll
@@ -536,41 +544,48 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     float m = -INFINITY, l = 0.f;
 
     const size_t khead = (size_t)kvh * page_size * DK, vhead = (size_t)kvh * page_size * DV;
-    uint4 kreg[NLK], vreg[NLV];
-    auto fetch = [&](int s) {
+    sp_v4u kreg0[NLK], vreg0[NLV], kreg1[NLK], vreg1[NLV];     // two steps' keys and values on their way: a load has two steps' time to arrive
+    int pgk[NLK], pgv[NLV];                            // page ids of the keys this thread fetches next: looked up a step ahead of the
+                                                       // fetch, so a step waits for one trip to memory, not for two in a row
+    auto key_of = [&](int s, int kk) -> int {
         int kb, klo, khi;
         step_of(s, kb, klo, khi);
+        int key = kb + kk;
+        key = key < klo ? klo : key;
+        return key > khi ? khi : key;
+    };
+    auto lookup = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < NLK; ++i) pgk[i] = bt[key_of(s, (tid + i * 256) / KCH) >> page_shift];
+#pragma unroll
+        for (int i = 0; i < NLV; ++i) pgv[i] = bt[key_of(s, (tid + i * 256) / VCH) >> page_shift];
+    };
+    auto fetch = [&](int s, sp_v4u* kreg, sp_v4u* vreg) {
 #pragma unroll
         for (int i = 0; i < NLK; ++i) {
             const int idx = tid + i * 256, kk = idx / KCH, c = idx - kk * KCH;
-            int key = kb + kk;
-            key = key < klo ? klo : key;
-            key = key > khi ? khi : key;
-            const int lp = key / page_size;
-            const size_t rowi = (size_t)bt[lp] * nkvh * page_size + (key - lp * page_size);
-            kreg[i] = *reinterpret_cast<const uint4*>(kcache + khead + rowi * DK + c * 8);
+            const int key = key_of(s, kk);
+            const size_t rowi = (((size_t)pgk[i] * nkvh) << page_shift) + (key & page_mask);
+            kreg[i] = *reinterpret_cast<const sp_v4u*>(kcache + khead + rowi * DK + c * 8);
         }
 #pragma unroll
         for (int i = 0; i < NLV; ++i) {
             const int idx = tid + i * 256, kk = idx / VCH, c = idx - kk * VCH;
-            int key = kb + kk;
-            key = key < klo ? klo : key;
-            key = key > khi ? khi : key;
-            const int lp = key / page_size;
-            const size_t rowi = (size_t)bt[lp] * nkvh * page_size + (key - lp * page_size);
-            vreg[i] = *reinterpret_cast<const uint4*>(vcache + vhead + rowi * DV + c * 8);
+            const int key = key_of(s, kk);
+            const size_t rowi = (((size_t)pgv[i] * nkvh) << page_shift) + (key & page_mask);
+            vreg[i] = *reinterpret_cast<const sp_v4u*>(vcache + vhead + rowi * DV + c * 8);
         }
     };
-    auto stash = [&]() {
+    auto stash = [&](const sp_v4u* kreg, const sp_v4u* vreg, uint16_t* Ks, uint16_t* Vs) {
 #pragma unroll
         for (int i = 0; i < NLK; ++i) {
             const int idx = tid + i * 256, kk = idx / KCH, c = idx - kk * KCH;
-            *reinterpret_cast<uint4*>(Ks + kk * PK + c * 8) = kreg[i];
+            *reinterpret_cast<sp_v4u*>(Ks + kk * PK + c * 8) = kreg[i];
         }
 #pragma unroll
         for (int i = 0; i < NLV; ++i) {
             const int idx = tid + i * 256, kk = idx / VCH, c = idx - kk * VCH;
-            *reinterpret_cast<uint4*>(Vs + kk * PV + c * 8) = vreg[i];
+            *reinterpret_cast<sp_v4u*>(Vs + kk * PV + c * 8) = vreg[i];
         }
     };
 
@@ -578,17 +593,19 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     const int vrow = 4 * half + ((lane & 15) >> 2);
     const int vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-    fetch(0);
-    for (int s = 0; s < n_steps; ++s) {
-        __syncthreads();                                   // the step before has been read
-        stash();
-        __syncthreads();
-        if (s + 1 < n_steps) fetch(s + 1);                 // in flight while this step is used
+    // Step s is fetched into registers three steps ahead and written to LDS one step ahead; its page ids are looked up a step before the fetch.
+    lookup(0);
+    fetch(0, kreg0, vreg0);
+    if (n_steps > 1) { lookup(1); fetch(1, kreg1, vreg1); }
+    stash(kreg0, vreg0, Ks0, Vs0);
+    if (n_steps > 2) { lookup(2); fetch(2, kreg0, vreg0); }
+    if (n_steps > 3) lookup(3);
+    auto compute = [&](int s, const uint16_t* Ks, const uint16_t* Vs) {
         int kb, klo, khi;
         step_of(s, kb, klo, khi);
-        if (!wave_ok || kb > wave_last) continue;          // nothing this wave may see
+        if (!wave_ok || kb > wave_last) return;            // nothing this wave may see
         const bool kept_run = s < kept_steps;
-        if (!kept_run && window > 0 && kb + kSpKeys - 1 < wave_first - window + 1 && kb >= keep_first) continue;   // all before this wave's windows, none kept
+        if (!kept_run && window > 0 && kb + kSpKeys - 1 < wave_first - window + 1 && kb >= keep_first) return;   // all before this wave's windows, none kept
 
         // ---- S^T = K Q^T : two tiles of 32 keys ----------------------------------
         sp_v16f sacc[2];
@@ -598,9 +615,8 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
             for (int r = 0; r < 16; ++r) sacc[tt][r] = 0.f;
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                SpFrag a;
-                a.u = *reinterpret_cast<const uint4*>(Ks + (32 * tt + lq) * PK + 16 * c + 8 * half);
-                sacc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[c].v, sacc[tt], 0, 0, 0);
+                const sp_bf16x8 a = *reinterpret_cast<const sp_bf16x8*>(Ks + (32 * tt + lq) * PK + 16 * c + 8 * half);
+                sacc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], sacc[tt], 0, 0, 0);
             }
         }
         // ---- mask: the run's bounds, the diagonal, the window and the kept first keys --------
@@ -656,12 +672,25 @@ attn_span_prefill_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
                 const uint16_t* vp = Vs + (16 * kc + vrow) * PV + 32 * dt + vcol;
-                SpFrag a;
-                a.h[0] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((sp_v4s __attribute__((address_space(3)))*)vp));
-                a.h[1] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((sp_v4s __attribute__((address_space(3)))*)(vp + 8 * PV)));
-                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b, oacc[dt], 0, 0, 0);
+                const sp_v4s lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((sp_v4s __attribute__((address_space(3)))*)vp);
+                const sp_v4s hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((sp_v4s __attribute__((address_space(3)))*)(vp + 8 * PV));
+                const sp_bf16x8 a = __builtin_bit_cast(sp_bf16x8, __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, oacc[dt], 0, 0, 0);
             }
         }
+    };
+    for (int s = 0; s < n_steps; s += 2) {
+        __syncthreads();                                   // stage 0 holds step s; stage 1 has been read
+        if (s + 1 < n_steps) stash(kreg1, vreg1, Ks1, Vs1);
+        if (s + 3 < n_steps) fetch(s + 3, kreg1, vreg1);
+        if (s + 4 < n_steps) lookup(s + 4);
+        compute(s, Ks0, Vs0);
+        if (s + 1 >= n_steps) break;
+        __syncthreads();                                   // stage 1 holds step s + 1; stage 0 has been read
+        if (s + 2 < n_steps) stash(kreg0, vreg0, Ks0, Vs0);
+        if (s + 4 < n_steps) fetch(s + 4, kreg0, vreg0);
+        if (s + 5 < n_steps) lookup(s + 5);
+        compute(s + 1, Ks1, Vs1);
     }
 
     if (!row_ok) return;
@@ -702,7 +731,7 @@ IC_EXPORT int ic_attn_span_prefill_supported(int dtype, int dk, int dv) {
     return dtype == IC_BF16 && span_dim_ok(dk) && span_dim_ok(dv);
 }
 
-// tiles: int32 [n_tiles, 4] = (request row, first token row, rows <= 128, first position).  Strides in elements; q rows, out rows and
+// tiles: int32 [n_tiles, 4] = (request row, first token row, rows <= 128, first position).  Pages of a power of two.  Strides in elements; q rows, out rows and
 // gate rows must start on 16-, 8- and 8-byte boundaries.  scale > 0.
 IC_EXPORT int ic_attn_span_prefill(const void* q, int q_stride, void* out, int out_stride, const void* gate, int gate_stride,
                                    int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride,
@@ -710,7 +739,9 @@ IC_EXPORT int ic_attn_span_prefill(const void* q, int q_stride, void* out, int o
                                    int window, int keep_first, int sink, hipStream_t stream) {
     if (n_tiles <= 0) return IC_OK;
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || window < 0 || keep_first < 0 || !(scale > 0.f)) return IC_ERR_ARG;
-    if (!ic_attn_span_prefill_supported(dtype, dk, dv)) return IC_ERR_UNSUPPORTED;
+    if (!ic_attn_span_prefill_supported(dtype, dk, dv) || (page_size & (page_size - 1))) return IC_ERR_UNSUPPORTED;
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
     if ((q_stride & 7) || (out_stride & 3) || (gate && (gate_stride & 3)) || ((uintptr_t)q & 15) || ((uintptr_t)out & 7) ||
         ((uintptr_t)gate & 7) || ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15))
         return IC_ERR_ARG;
@@ -721,7 +752,7 @@ IC_EXPORT int ic_attn_span_prefill(const void* q, int q_stride, void* out, int o
     if (dk == K && dv == V) {                                                                                                 \
         hipLaunchKernelGGL((attn_span_prefill_kernel<K, V>), grid, block, 0, stream, (const uint16_t*)q, q_stride,            \
                            (uint16_t*)out, out_stride, (const uint16_t*)gate, gate_stride, (const uint16_t*)kcache,           \
-                           (const uint16_t*)vcache, block_tables, bt_stride, (const int4*)tiles, nh, nkvh, page_size, c,      \
+                           (const uint16_t*)vcache, block_tables, bt_stride, (const int4*)tiles, nh, nkvh, page_shift, c,      \
                            window, keep_first, sink);                                                                         \
         return ic_launch_status();                                                                                            \
     }

@@ -112,7 +112,7 @@ IC_EXPORT int ic_norm_into_stream(const void* y, int y_dtype, const float* bias,
 //                mix_mode 2: v = (1 - lambda) v + lambda v_keep[t]        -> V plane at slots[t]
 // norm_mode 0: none; 1: every head's dk entries to unit root mean square, times w[dk] (shared by the heads);
 // 2: the whole of q (or k) to unit root mean square, times w[nh * dk] (or w[nkvh * dk]).
-// One block per token, the row in LDS as float32 (dynamic, (nh + nkvh) * dk + nkvh * dv floats).
+// One wave per (token, head of q, k or v); head sizes up to 512.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -121,58 +121,60 @@ qk_norm_store_kernel(const T* __restrict__ rows, int row_stride, const float* __
                      int mix_mode, const float* __restrict__ lambda, float* __restrict__ v_keep,
                      T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache,
                      const int* __restrict__ slots, int nh, int nkvh, int dk, int dv, int page_size) {
-    extern __shared__ float row[];
-    __shared__ float red[16];
-    __shared__ float head_r[512];
-    const int t = blockIdx.x, tid = threadIdx.x;
-    const int nq = nh * dk, nk = nkvh * dk, nv = nkvh * dv, n = nq + nk + nv;
+    // Grid (tokens, ceil(heads / 4)): one wave per head of q, k or v; a lane holds up to 8 of the head's entries.
+    const int t = blockIdx.x, lane = threadIdx.x & 63;
+    const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (head >= nh + 2 * nkvh) return;
+    const int nq = nh * dk, nk = nkvh * dk, nv = nkvh * dv;
     const T* src = rows + (size_t)t * row_stride;
-    for (int i = tid; i < n; i += blockDim.x) row[i] = to_f32(src[i]) + (bias ? bias[i] : 0.f);
-    __syncthreads();
     const int slot = slots ? slots[t] : -1;
     const int pg = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - pg * page_size : 0;
-
-    if (norm_mode == 1) {
-        // one wave per head, heads of q and k alike
-        const int lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
-        for (int h = wave; h < nh + nkvh; h += nw) {
+    float val[8];
+    if (head < nh + nkvh) {                               // a head of q or k
+        const bool is_q = head < nh;
+        const int base = head * dk;                       // k follows q in the row
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int e = lane + 64 * j;
+            val[j] = e < dk ? to_f32(src[base + e]) + (bias ? bias[base + e] : 0.f) : 0.f;
+        }
+        const float* w = is_q ? qw : kw;
+        if (norm_mode == 1) {
             float ss = 0.f;
-            for (int j = lane; j < dk; j += 64) { const float v = row[h * dk + j]; ss += v * v; }
-            ss = wave_sum(ss);
-            if (lane == 0) head_r[h] = 1.0f / sqrtf(ss / (float)dk + eps);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss += val[j] * val[j];
+            const float r = 1.0f / sqrtf(wave_sum(ss) / (float)dk + eps);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { const int e = lane + 64 * j; if (e < dk) val[j] = val[j] * r * w[e]; }
+        } else if (norm_mode == 2) {                      // the sum runs over the whole of q (or k), which every wave reads
+            const int p0 = is_q ? 0 : nq, pn = is_q ? nq : nk;
+            float ss = 0.f;
+            for (int i = lane; i < pn; i += 64) { const float v = to_f32(src[p0 + i]) + (bias ? bias[p0 + i] : 0.f); ss += v * v; }
+            const float r = 1.0f / sqrtf(wave_sum(ss) / (float)pn + eps);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { const int e = lane + 64 * j; if (e < dk) val[j] = val[j] * r * w[base - p0 + e]; }
         }
-        __syncthreads();
-        for (int i = tid; i < nq + nk; i += blockDim.x) {
-            const int h = i / dk, j = i - h * dk;
-            row[i] = row[i] * head_r[h] * (h < nh ? qw[j] : kw[j]);
+        T* dst = nullptr;
+        if (is_q) dst = q_out + (size_t)t * nq + base;
+        else if (slot >= 0 && kcache) dst = kcache + (((size_t)pg * nkvh + (head - nh)) * page_size + off) * dk;
+        if (dst) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) { const int e = lane + 64 * j; if (e < dk) dst[e] = from_f32<T>(val[j]); }
         }
-    } else if (norm_mode == 2) {
-        float sq = 0.f, sk = 0.f;
-        for (int i = tid; i < nq; i += blockDim.x) sq += row[i] * row[i];
-        for (int i = nq + tid; i < nq + nk; i += blockDim.x) sk += row[i] * row[i];
-        sq = block_sum(sq, red);
-        sk = block_sum(sk, red);
-        const float rq = 1.0f / sqrtf(sq / (float)nq + eps), rk = 1.0f / sqrtf(sk / (float)nk + eps);
-        for (int i = tid; i < nq; i += blockDim.x) row[i] = row[i] * rq * qw[i];
-        for (int i = tid; i < nk; i += blockDim.x) row[nq + i] = row[nq + i] * rk * kw[i];
+        return;
     }
-    __syncthreads();
-    for (int i = tid; i < nq; i += blockDim.x) q_out[(size_t)t * nq + i] = from_f32<T>(row[i]);
-    if (slot >= 0 && kcache) {
-        for (int i = tid; i < nk; i += blockDim.x) {
-            const int h = i / dk, j = i - h * dk;
-            kcache[(((size_t)pg * nkvh + h) * page_size + off) * dk + j] = from_f32<T>(row[nq + i]);
-        }
-    }
+    const int vh = head - nh - nkvh, base = nq + nk + vh * dv;
     const float lam = (mix_mode == 2) ? lambda[0] : 0.f;
-    for (int i = tid; i < nv; i += blockDim.x) {
-        float v = row[nq + nk + i];
-        if (mix_mode == 1) v_keep[(size_t)t * nv + i] = v;
-        else if (mix_mode == 2) v = (1.0f - lam) * v + lam * v_keep[(size_t)t * nv + i];
-        if (slot >= 0 && vcache) {
-            const int h = i / dv, j = i - h * dv;
-            vcache[(((size_t)pg * nkvh + h) * page_size + off) * dv + j] = from_f32<T>(v);
-        }
+    T* dst = (slot >= 0 && vcache) ? vcache + (((size_t)pg * nkvh + vh) * page_size + off) * dv : nullptr;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int e = lane + 64 * j;
+        if (e >= dv) continue;
+        float v = to_f32(src[base + e]) + (bias ? bias[base + e] : 0.f);
+        float* keep = v_keep + (size_t)t * nv + vh * dv + e;
+        if (mix_mode == 1) *keep = v;
+        else if (mix_mode == 2) v = (1.0f - lam) * v + lam * *keep;
+        if (dst) dst[e] = from_f32<T>(v);
     }
 }
 
@@ -184,15 +186,14 @@ IC_EXPORT int ic_qk_norm_store(const void* rows, int row_stride, int dtype, cons
     if (nh <= 0 || nkvh <= 0 || dk <= 0 || dv <= 0 || page_size <= 0 || norm_mode < 0 || norm_mode > 2 || mix_mode < 0 ||
         mix_mode > 2)
         return IC_ERR_ARG;
-    if (nh + nkvh > 512) return IC_ERR_TOO_LARGE;
     if (norm_mode != 0 && (qw == nullptr || kw == nullptr)) return IC_ERR_ARG;
     if (mix_mode != 0 && v_keep == nullptr) return IC_ERR_ARG;
     if (mix_mode == 2 && lambda == nullptr) return IC_ERR_ARG;
     const long long n = (long long)(nh + nkvh) * dk + (long long)nkvh * dv;
     if (row_stride < n) return IC_ERR_ARG;
-    const size_t lds = (size_t)n * sizeof(float);
-    if (lds > 60 * 1024) return IC_ERR_TOO_LARGE;
-    dim3 grid(T), block(256);
+    if (dk > 512 || dv > 512) return IC_ERR_TOO_LARGE;
+    const size_t lds = 0;
+    dim3 grid(T, (nh + 2 * nkvh + 3) / 4), block(256);
     if (dtype == IC_F32)
         hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, lds, stream, (const float*)rows, row_stride, bias, qw,
                            kw, norm_mode, eps, mix_mode, lambda, v_keep, (float*)q_out, (float*)kcache, (float*)vcache,

@@ -149,7 +149,8 @@ class SpanAttention(Mixer):
         n_dec, n_tiles = ctx.n_decode_rows, ctx.n_prefill_tiles
         tiled = rt.attention_impl == "auto" and n_dec + n_tiles > 0
         use_dec = tiled and n_dec > 0 and ops.attention_span_decode_supported(rt.dtype, self.dk, self.dv)
-        use_pre = tiled and n_tiles > 0 and self.scale > 0 and ops.attention_span_prefill_supported(rt.dtype, self.dk, self.dv)
+        use_pre = (tiled and n_tiles > 0 and self.scale > 0 and ctx.page_size & (ctx.page_size - 1) == 0
+                   and ops.attention_span_prefill_supported(rt.dtype, self.dk, self.dv))
         if not (use_dec or n_dec == 0) or not (use_pre or n_tiles == 0) or not tiled:
             ops.attention_span_generic(q, out, gate, cache.k, cache.v, cache.block_tables, ctx.token_req, ctx.positions, *args)
             return
