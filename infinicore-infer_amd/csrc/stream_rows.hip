@@ -12,6 +12,33 @@
 // [num_pages, n_kv_heads, page_size, value_dim].
 #include "common.h"
 
+// 16 bytes of a row as float32 values.
+template <typename T> struct RowPack;
+template <> struct RowPack<float> {
+    static constexpr int N = 4;
+    __device__ static void load(const float* p, float* o) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+    __device__ static void store(float* p, const float* o) { *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]); }
+};
+template <> struct RowPack<bf16> {
+    static constexpr int N = 8;
+    __device__ static void load(const bf16* p, float* o) {
+        typedef unsigned v4u __attribute__((ext_vector_type(4)));
+        const v4u v = *reinterpret_cast<const v4u*>(p);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(v[i] << 16); o[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u); }
+    }
+    __device__ static void store(bf16* p, const float* o) {
+        typedef unsigned v4u __attribute__((ext_vector_type(4)));
+        v4u v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = (uint32_t)f32_to_bf16_bits(o[2 * i]) | ((uint32_t)f32_to_bf16_bits(o[2 * i + 1]) << 16);
+        *reinterpret_cast<v4u*>(p) = v;
+    }
+};
+
 // ---------------------------------------------------------------------------------------------
 // x[t, 2i] = table[tok, 2i] * scale + sin(p f_i), x[t, 2i+1] = table[tok, 2i+1] * scale + cos(p f_i);
 // f_i is a float32 table [d/2] made by the host; the angle is the float32 product p * f_i.
@@ -178,6 +205,89 @@ qk_norm_store_kernel(const T* __restrict__ rows, int row_stride, const float* __
     }
 }
 
+// The same work 16 bytes a lane, for head sizes whose 16-byte pieces are a power of two per head (LPH lanes share a head of
+// q or k, LPV lanes a head of v) and rows that start on 16-byte boundaries.  Grid (tokens, ceil(items / 256)); an item is one
+// 16-byte piece of the row [q | k | v].  norm_mode 1: the lanes of a head sum their squares among themselves; norm_mode 2: every
+// wave sums the whole of q (or k) first.  A wave never straddles q/k and v pieces (the launcher pads the q/k pieces to whole waves).
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_store_vec_kernel(const T* __restrict__ rows, int row_stride, const float* __restrict__ bias,
+                         const float* __restrict__ qw, const float* __restrict__ kw, int norm_mode, float eps,
+                         int mix_mode, const float* __restrict__ lambda, float* __restrict__ v_keep,
+                         T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache,
+                         const int* __restrict__ slots, int nh, int nkvh, int dk, int dv, int page_size, int qk_items_padded) {
+    constexpr int N = RowPack<T>::N;
+    const int t = blockIdx.x, lane = threadIdx.x & 63;
+    const int item = blockIdx.y * 256 + threadIdx.x;
+    const int nq = nh * dk, nk = nkvh * dk, nv = nkvh * dv;
+    const int lph = dk / N, lpv = dv / N;
+    const T* src = rows + (size_t)t * row_stride;
+    const int slot = slots ? slots[t] : -1;
+    const int pg = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - pg * page_size : 0;
+    float val[N];
+    if (item < qk_items_padded) {                         // (wave-uniform) pieces of q and k
+        const bool live = item < (nq + nk) / N;
+        const int e0 = live ? item * N : 0;               // first entry of the piece in [q | k]
+        const int head = e0 / dk, j0 = e0 - head * dk;
+        const bool is_q = head < nh;
+        RowPack<T>::load(src + e0, val);
+        if (bias) {
+#pragma unroll
+            for (int i = 0; i < N; ++i) val[i] += bias[e0 + i];
+        }
+        const float* w = is_q ? qw : kw;
+        if (norm_mode == 1) {
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < N; ++i) ss += val[i] * val[i];
+            for (int o = 1; o < lph; o <<= 1) ss += __shfl_xor(ss, o, kWave);       // lph is a power of two and divides 64
+            const float r = 1.0f / sqrtf(ss / (float)dk + eps);
+#pragma unroll
+            for (int i = 0; i < N; ++i) val[i] = val[i] * r * w[j0 + i];
+        } else if (norm_mode == 2) {
+            // a wave's pieces may belong to q and to k: both sums are formed by every wave
+            float sq = 0.f, sk = 0.f;
+            for (int i = lane * N; i < nq + nk; i += 64 * N) {
+                float v[N];
+                RowPack<T>::load(src + i, v);
+                float s2 = 0.f;
+#pragma unroll
+                for (int e = 0; e < N; ++e) { const float z = v[e] + (bias ? bias[i + e] : 0.f); s2 += z * z; }
+                if (i < nq) sq += s2; else sk += s2;
+            }
+            sq = wave_sum(sq);
+            sk = wave_sum(sk);
+            const float r = is_q ? 1.0f / sqrtf(sq / (float)nq + eps) : 1.0f / sqrtf(sk / (float)nk + eps);
+            const int wj = is_q ? e0 : e0 - nq;
+#pragma unroll
+            for (int i = 0; i < N; ++i) val[i] = val[i] * r * w[wj + i];
+        }
+        if (!live) return;
+        if (is_q) RowPack<T>::store(q_out + (size_t)t * nq + e0, val);
+        else if (slot >= 0 && kcache)
+            RowPack<T>::store(kcache + (((size_t)pg * nkvh + (head - nh)) * page_size + off) * dk + j0, val);
+        return;
+    }
+    const int vi = item - qk_items_padded;
+    if (vi >= nv / N) return;
+    const int e0 = vi * N, vh = e0 / dv, j0 = e0 - vh * dv;
+    RowPack<T>::load(src + nq + nk + e0, val);
+    if (bias) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) val[i] += bias[nq + nk + e0 + i];
+    }
+    if (mix_mode == 1) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) v_keep[(size_t)t * nv + e0 + i] = val[i];
+    } else if (mix_mode == 2) {
+        const float lam = lambda[0];
+#pragma unroll
+        for (int i = 0; i < N; ++i) val[i] = (1.0f - lam) * val[i] + lam * v_keep[(size_t)t * nv + e0 + i];
+    }
+    if (slot >= 0 && vcache) RowPack<T>::store(vcache + (((size_t)pg * nkvh + vh) * page_size + off) * dv + j0, val);
+    (void)lpv;
+}
+
 IC_EXPORT int ic_qk_norm_store(const void* rows, int row_stride, int dtype, const float* bias, const float* qw,
                                const float* kw, int norm_mode, float eps, int mix_mode, const float* lambda,
                                float* v_keep, void* q_out, void* kcache, void* vcache, const int* slots, int T, int nh,
@@ -193,6 +303,29 @@ IC_EXPORT int ic_qk_norm_store(const void* rows, int row_stride, int dtype, cons
     if (row_stride < n) return IC_ERR_ARG;
     if (dk > 512 || dv > 512) return IC_ERR_TOO_LARGE;
     const size_t lds = 0;
+    {
+        // 16 bytes a lane where the sizes allow it: pieces per head of q/k a power of two that divides 64, values in whole pieces,
+        // rows, outputs and cache rows on 16-byte boundaries
+        const int pack = dtype == IC_F32 ? 4 : 8;
+        const int lph = dk % pack == 0 ? dk / pack : 0;
+        const bool pow2 = lph > 0 && lph <= 64 && (lph & (lph - 1)) == 0;
+        const uintptr_t ptrs = (uintptr_t)rows | (uintptr_t)q_out | (uintptr_t)kcache | (uintptr_t)vcache;
+        if ((dtype == IC_F32 || dtype == IC_BF16) && pow2 && dv % pack == 0 && row_stride % pack == 0 && (ptrs & 15) == 0) {
+            const int qk_items = (int)(((long long)(nh + nkvh) * dk) / pack);
+            const int qk_padded = (qk_items + 63) / 64 * 64;
+            const int items = qk_padded + nkvh * dv / pack;
+            dim3 vgrid(T, (items + 255) / 256), vblock(256);
+            if (dtype == IC_F32)
+                hipLaunchKernelGGL(qk_norm_store_vec_kernel<float>, vgrid, vblock, 0, stream, (const float*)rows, row_stride, bias, qw,
+                                   kw, norm_mode, eps, mix_mode, lambda, v_keep, (float*)q_out, (float*)kcache, (float*)vcache, slots,
+                                   nh, nkvh, dk, dv, page_size, qk_padded);
+            else
+                hipLaunchKernelGGL(qk_norm_store_vec_kernel<bf16>, vgrid, vblock, 0, stream, (const bf16*)rows, row_stride, bias, qw, kw,
+                                   norm_mode, eps, mix_mode, lambda, v_keep, (bf16*)q_out, (bf16*)kcache, (bf16*)vcache, slots, nh,
+                                   nkvh, dk, dv, page_size, qk_padded);
+            return ic_launch_status();
+        }
+    }
     dim3 grid(T, (nh + 2 * nkvh + 3) / 4), block(256);
     if (dtype == IC_F32)
         hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, lds, stream, (const float*)rows, row_stride, bias, qw,
@@ -223,9 +356,34 @@ __global__ void activation_kernel(const T* __restrict__ in, T* __restrict__ out,
         out[i] = from_f32<T>(act_apply(to_f32(in[i]), kind));
 }
 
+// 16 bytes a thread (n a multiple of the pack, both pointers on 16-byte boundaries).
+template <typename T>
+__global__ void activation_vec_kernel(const T* __restrict__ in, T* __restrict__ out, long long n_packs, int kind) {
+    constexpr int N = RowPack<T>::N;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n_packs; i += stride) {
+        float v[N];
+        RowPack<T>::load(in + i * N, v);
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] = act_apply(v[e], kind);
+        RowPack<T>::store(out + i * N, v);
+    }
+}
+
 IC_EXPORT int ic_activation(const void* in, void* out, int dtype, long long n, int kind, hipStream_t stream) {
     if (n <= 0) return IC_OK;
     if (kind < 0 || kind > 2) return IC_ERR_ARG;
+    const int pack = dtype == IC_F32 ? 4 : 8;
+    if ((dtype == IC_F32 || dtype == IC_BF16) && n % pack == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
+        const long long np = n / pack;
+        long long vb = (np + 255) / 256;
+        if (vb > 8192) vb = 8192;
+        if (dtype == IC_F32)
+            hipLaunchKernelGGL(activation_vec_kernel<float>, dim3((unsigned)vb), dim3(256), 0, stream, (const float*)in, (float*)out, np, kind);
+        else
+            hipLaunchKernelGGL(activation_vec_kernel<bf16>, dim3((unsigned)vb), dim3(256), 0, stream, (const bf16*)in, (bf16*)out, np, kind);
+        return ic_launch_status();
+    }
     long long blocks = (n + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     dim3 grid((unsigned)blocks), block(256);
