@@ -129,6 +129,8 @@ class FopezenConfig:
     def max_positions(self) -> int:
         return self.context_cap if self.context_cap is not None else DEFAULT_CONTEXT
 
+    context_is_open = True      # positions are bounded by the serving cap or the cache pool only
+
     @property
     def default_dtype(self) -> str:
         return "bfloat16"

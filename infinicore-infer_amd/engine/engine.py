@@ -154,6 +154,10 @@ class Engine:
                  **kw):
         """``dtype`` None: the checkpoint's own (config.json's torch_dtype; float16 runs as bfloat16)."""
         cfg = config_from_dir(model_dir, max_tokens=max_context) if max_context else config_from_dir(model_dir)
+        if (not max_context and max_tokens and getattr(cfg, "context_is_open", False)
+                and int(max_tokens) > cfg.max_positions):
+            # a design without a context limit of its own: a pool larger than its default context lifts the limit to the pool
+            cfg = config_from_dir(model_dir, max_tokens=int(max_tokens))
         if dtype is None:
             dtype = getattr(torch, getattr(cfg, "default_dtype", "bfloat16"))
         rt = Runtime(dtype=dtype, device=device, attention_impl=attention_impl, gemm_impl=gemm_impl)

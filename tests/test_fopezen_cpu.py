@@ -30,6 +30,7 @@ def test_config_to_model_spec():
     assert spec.embedding.params["sinusoid_base"] == 10000.0 and spec.head.params["tensor"] == "embed"
     assert config_from_dict(cfg.to_dict()).model_spec().layers[2].mixer.params == spec.layers[2].mixer.params
     assert config_from_dict(F1, max_tokens=300).max_positions == 300
+    assert cfg.context_is_open and cfg.max_positions == 65536
 
 
 @pytest.mark.parametrize("change,what", [

@@ -45,8 +45,14 @@ F3 = {"architecture": "Fopezen", "vocab": 300, "width": 192, "norm": {"eps": 1e-
     _layer("attention_2", 8, 2, 64, 64, 0.12, 130, 0, False, 256),
     _layer("attention", 8, 1, 32, 128, 0.2, 64, 16, True, None),
 ]}
-CONFIGS = {"F1": F1, "F2": F2, "F3": F3}
-LENGTHS = {"F1": [1, 2, 130, 61, 210, 37], "F2": [3, 75, 1, 140, 18, 66], "F3": [5, 260, 129, 64, 331, 2]}
+# F4: no masks at all (every key is read, nothing is given back: decoding may run a step ahead of the host), no value mixing.
+F4 = {"architecture": "Fopezen", "vocab": 150, "width": 64, "norm": {"eps": 1e-5}, "layers": [
+    _layer("attention", 2, 2, 32, 32, 0.18, None, 0, False, 96),
+    _layer("attention_2", 4, 1, 16, 24, 0.25, None, 0, False, 80),
+]}
+CONFIGS = {"F1": F1, "F2": F2, "F3": F3, "F4": F4}
+LENGTHS = {"F1": [1, 2, 130, 61, 210, 37], "F2": [3, 75, 1, 140, 18, 66], "F3": [5, 260, 129, 64, 331, 2],
+           "F4": [2, 90, 17, 1, 133, 40]}
 
 
 def _write_model(folder, cfg, seed):
@@ -379,7 +385,7 @@ def _plain_greedy(cfg, W, prompt, n):
     return toks[len(prompt):]
 
 
-@pytest.mark.parametrize("name", ["F1", "F2"])
+@pytest.mark.parametrize("name", ["F1", "F2", "F4"])
 def test_greedy_generation_through_the_entry_point_and_scheduler(tmp_path_factory, name):
     """Several prompts of unequal length through CausalLM.generate_batch (the scheduler: chunked prompts, continuous
     batching, recorded decode steps) in float32: the plain implementation's greedy tokens."""
@@ -392,6 +398,8 @@ def test_greedy_generation_through_the_entry_point_and_scheduler(tmp_path_factor
     for p, o in zip(prompts, outs):
         assert o == _plain_greedy(cfg, W, p, 12)
     model.engine.cache.check_invariants()
+    if name == "F4":
+        assert model.engine.steps_ahead > 0          # without windows the device fed its own tokens to recorded steps
 
 
 def test_command_line_runs_the_design(tmp_path_factory):
