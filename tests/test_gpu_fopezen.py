@@ -414,3 +414,43 @@ def test_command_line_runs_the_design(tmp_path_factory):
     assert r.returncode == 0, r.stderr[-2000:]
     want = _plain_greedy(F1, W, prompt, 6)
     assert " ".join(map(str, want)) in " ".join(r.stdout.split()), r.stdout[-2000:]
+
+
+# ---- configurations drawn from seeds -------------------------------------------------------------------------------------
+def _drawn_config(seed):
+    """Layer order, sizes (also ones that are no multiple of 8 or 16), windows, kept keys, scales and mixing drawn from a seed."""
+    rng = random.Random(seed)
+    width = rng.choice([34, 48, 64, 100, 136])
+    kv, vdim = rng.choice([1, 2, 3]), rng.choice([8, 12, 20, 32, 64])        # shared by the mixing layers
+    layers = []
+    for i in range(rng.choice([2, 3, 4, 5])):
+        mixes = rng.random() < 0.6
+        g = kv if mixes else rng.choice([1, 2, 4])
+        heads = g * rng.choice([1, 2, 3, 5])
+        dim = rng.choice([8, 12, 16, 24, 32, 40, 64, 128])
+        dv = vdim if mixes else rng.choice([8, 16, 32, 48, 64, 128])
+        size = rng.choice([None, 1, 2, 7, 16, 31, 64, 65, 100])
+        keep = rng.choice([0, 0, 1, 3, 16, 17, 70]) if size else 0
+        ff = rng.choice([None, 24, 50, 128])
+        layers.append(_layer(rng.choice(["attention", "attention_2"]), heads, g, dim, dv, round(rng.uniform(0.05, 0.4), 3),
+                             size, keep, mixes, ff))
+    return {"architecture": "Fopezen", "vocab": rng.choice([53, 128, 301]), "width": width,
+            "norm": {"eps": rng.choice([1e-5, 1e-6, 1e-3])}, "layers": layers}
+
+
+@pytest.mark.parametrize("seed", list(range(10)))
+def test_drawn_configurations(tmp_path_factory, seed):
+    from infinicore_infer_amd.engine import Engine
+    cfg = _drawn_config(seed)
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "fopezen_drawn_%d" % seed)
+    W = _write_model(folder, cfg, seed)
+    rng = random.Random(seed + 100)
+    requests = {"r%d" % i: H.random_tokens(cfg["vocab"], n, seed * 10 + i)
+                for i, n in enumerate([rng.choice([1, 2, 5, 40, 66, 129, 180, 250]) for _ in range(5)])}
+    ref = {rid: P.forward(cfg, W, toks, torch.float64) for rid, toks in requests.items()}
+    steps, max_tokens = H.trace_mixed(requests, seed=seed)
+    for dname, dtype, tol in DTYPES:
+        engine = Engine.from_dir(folder, dtype=dtype, max_tokens=max_tokens, page_size=16, max_requests=4)
+        H.compare(H.run_trace(engine, steps), ref, tol, "drawn %d %s" % (seed, dname), steps)
+        engine.cache.check_invariants()
+        assert not engine.cache.requests
