@@ -73,7 +73,15 @@ struct NormFuse {
     const float* g;            // [N]
     float rscale;
     float* ss_out;             // [gridDim.x, 16]
+    int act;                   // plain store only: 0 none, else the product (rounded to its type first, as when stored) goes
+                               // through an activation: 1 relu(z)^2, 2 gelu_tanh(z), 3 silu(z)
 };
+
+__device__ __forceinline__ float gemm_act(float z, int act) {
+    if (act == 1) { const float r = fmaxf(z, 0.f); return r * r; }
+    if (act == 2) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    return z / (1.0f + expf(-z));
+}
 
 // lane i of a row of 16 lanes takes the value of lane (i + S) % 16 (a DPP row rotation, no LDS)
 template <int S> __device__ __forceinline__ v4s row_from_above(v4s v) {
@@ -450,7 +458,10 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 #pragma unroll
                 for (int w = 0; w < WPB - 1; ++w) v += red[w][nt * MT + mt][lane][e];
                 const int n = n0 + 16 * nt + 4 * kq + e;    // row i of D
-                if (m < M && n < N) C[(size_t)m * ldc + n] = from_f32<TC>(alpha * v);
+                if (m < M && n < N) {
+                    if (nf.act) C[(size_t)m * ldc + n] = from_f32<TC>(gemm_act(to_f32(from_f32<TC>(alpha * v)), nf.act));
+                    else C[(size_t)m * ldc + n] = from_f32<TC>(alpha * v);
+                }
             }
         }
 }
@@ -647,7 +658,10 @@ gemm_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int n = tile * 16 + 4 * kq + e;
-                if (n < N) C[(size_t)r * ldc + n] = from_f32<TC>(scale * v[e]);
+                if (n < N) {
+                    if (nf.act) C[(size_t)r * ldc + n] = from_f32<TC>(gemm_act(to_f32(from_f32<TC>(scale * v[e])), nf.act));
+                    else C[(size_t)r * ldc + n] = from_f32<TC>(scale * v[e]);
+                }
             }
         }
     };
@@ -861,6 +875,7 @@ IC_EXPORT int ic_gemm_nt_residual_parts(int N) {
     return (N + cols - 1) / cols;
 }
 
+// c_mode 3, 4, 5: as 0 with an activation on the stored value, C = act(alpha * A W^T): relu(z)^2, gelu_tanh(z), silu(z).
 // c_mode 0: C [M, N] = alpha * A W^T.  c_mode 1 (M <= 16, N even, alpha ignored): W = [gate; up] and
 // C [M, N/2] = up * silu(gate), both projections rounded to C's type before the activation.
 // c_mode 2 (M <= 16, bfloat16 C, `tail` given): x += tail->alpha * (alpha * A W^T); C = x * tail->weight;
@@ -870,12 +885,13 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
                          int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode,
                          const IcRowFactor* row_factor, const IcResidualNorm* tail, hipStream_t stream) {
     if (M <= 0 || N <= 0) return IC_OK;
-    if (K <= 0 || lda < K || ldw < K || c_mode < 0 || c_mode > 2) return IC_ERR_ARG;
+    if (K <= 0 || lda < K || ldw < K || c_mode < 0 || c_mode > 5) return IC_ERR_ARG;
     if (c_mode == 1 ? ((N & 1) || ldc < N / 2) : (ldc < N)) return IC_ERR_ARG;
     if ((c_mode == 2) != (tail != nullptr)) return IC_ERR_ARG;
     if (!ic_gemm_nt_supported(a_dtype, w_dtype, c_dtype)) return IC_ERR_UNSUPPORTED;
     if ((M + 63) / 64 > 65535) return IC_ERR_ARG;
     NormFuse nf{};
+    if (c_mode >= 3) { nf.act = c_mode - 2; c_mode = 0; }      // the plain product with an activation on its way out
     if (!norm_fuse_args(row_factor, tail, M, N, K, c_dtype, ic_gemm_nt_residual_parts(N), nf)) return IC_ERR_ARG;
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
     if (c_mode == 1 && M > 16 && (M > 32 || c_dtype != IC_BF16 || row_factor || !lines_apply(aligned, K))) return IC_ERR_ARG;

@@ -112,7 +112,8 @@ typedef struct {
 } IcResidualNorm;
 // C[M, N] = alpha * A[M, K] W[N, K]^T, bfloat16 operands, float32 accumulation.  c_mode 1 (M <= 16):
 // W = [gate; up], C[M, N/2] = up * silu(gate).  c_mode 2 (M <= 16, bfloat16 C, tail != NULL):
-// x += tail->alpha * (alpha A W^T), C = x * tail->weight.  row_factor (nullable, M <= 16): see above.
+// x += tail->alpha * (alpha A W^T), C = x * tail->weight.  c_mode 3 / 4 / 5: C = act(alpha A W^T) with act = relu(z)^2 /
+// gelu_tanh(z) / silu(z), applied to the product as rounded to C's type.  row_factor (nullable, M <= 16): see above.
 int ic_gemm_nt_supported(int a_dtype, int w_dtype, int c_dtype);
 int ic_gemm_nt_residual_parts(int N);
 int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode, const IcRowFactor* row_factor, const IcResidualNorm* tail, hipStream_t stream);

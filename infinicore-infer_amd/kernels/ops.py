@@ -436,7 +436,8 @@ def gemm_epilogue_rows(kind: str, a, w) -> int:
     return int(get_lib().ic_gemm_nt_epilogue_rows({"swiglu": 1, "rope": 2}[kind], int(a.shape[1]), int(a.stride(0)), int(w.stride(0))))
 
 
-def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_factor=None, residual=None, whole_lines: bool = True):
+def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_factor=None, residual=None, whole_lines: bool = True,
+            activation=None):
     """out[M, N] = alpha * a[M, K] @ w[N, K]^T (bfloat16 operands, float32 accumulation).
     swiglu_output (M <= gemm_epilogue_rows("swiglu", a, w)): w = [gate rows; up rows] and out[M, N/2] = up * silu(gate).
     row_factor = (sumsq [n_parts, 16], width, eps), M <= 16: row m of the product is first multiplied by
@@ -444,7 +445,8 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_fact
     residual = (x float32 [M, N], weight float32 [N], beta, sumsq_out float32 [residual_parts(N), 16]),
     M <= 16, bfloat16 out: x += beta * (the product rounded to bfloat16); out = x * weight;
     sumsq_out[b, m] = sum of x[m]^2 over columns 16 b .. 16 b + 15.
-    whole_lines False (tests): the weights are loaded in operand layout also where whole cache lines would apply."""
+    whole_lines False (tests): the weights are loaded in operand layout also where whole cache lines would apply.
+    activation ("relu2", "gelu_tanh", "silu"; not with the other epilogues): out = act(the product as rounded to out's dtype)."""
     import ctypes
     _dev(a, w, out)
     M, K = a.shape
@@ -466,6 +468,9 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_fact
               "gemm_nt: sumsq_out must be float32 [residual_parts(N) <= 256, 16]")
         rn = IcResidualNorm(x.data_ptr(), x.stride(0), weight.data_ptr(), float(beta), sumsq_out.data_ptr(), sumsq_out.shape[0])
         mode = 2
+    if activation is not None:
+        _need(mode == 0 and activation in ACTIVATIONS, "gemm_nt: an activation goes with the plain product only (have %s)" % ", ".join(sorted(ACTIVATIONS)))
+        mode = 3 + ACTIVATIONS[activation]
     if not whole_lines:
         check(get_lib().ic_gemm_nt_variant(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), dtype_code(w.dtype),
                                            out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),

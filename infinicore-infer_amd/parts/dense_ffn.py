@@ -1,9 +1,11 @@
 """Dense feed-forward with one up projection: down(act(up h)), no gate and no biases.
-``activation``: "relu2" (the square of relu), "gelu_tanh" or "silu"; computed in float32 inside the kernel."""
+``activation``: "relu2" (the square of relu), "gelu_tanh" or "silu"; computed in float32 inside the kernel.  For few rows
+the activation is the epilogue of the up projection (applied to the product as rounded to its dtype, so the result is the
+same bits as the product followed by the activation kernel)."""
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import FeedForward, register_part
-from .linear import linear
+from .linear import linear, own_kernel_applies
 
 
 @register_part("feed_forward", "dense_act")
@@ -31,8 +33,11 @@ class DenseActFeedForward(FeedForward):
         rt = self.runtime
         T = h.shape[0]
         u = ctx.ws.buffer("ffn_up", (T, self.intermediate_size), rt.dtype)
-        linear(h, self.w_up, u, rt.gemm_impl, ws=ctx.ws)
-        ops.activation(u, u, self.activation)
+        if h.dtype == self.w_up.dtype and own_kernel_applies(T, h.dtype, self.w_up.dtype, u.dtype, rt.gemm_impl):
+            ops.gemm_nt(h, self.w_up, u, activation=self.activation)      # few rows: the activation is the product's epilogue
+        else:
+            linear(h, self.w_up, u, rt.gemm_impl, ws=ctx.ws)
+            ops.activation(u, u, self.activation)
         y = ctx.ws.buffer("ffn_out", (T, self.hidden_size), rt.dtype)
         linear(u, self.w_down, y, rt.gemm_impl, ws=ctx.ws)
         return y

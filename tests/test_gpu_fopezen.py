@@ -454,3 +454,18 @@ def test_drawn_configurations(tmp_path_factory, seed):
         H.compare(H.run_trace(engine, steps), ref, tol, "drawn %d %s" % (seed, dname), steps)
         engine.cache.check_invariants()
         assert not engine.cache.requests
+
+
+@pytest.mark.parametrize("kind", ["relu2", "gelu_tanh", "silu"])
+@pytest.mark.parametrize("M,N,K", [(1, 384, 256), (8, 14336, 4096), (16, 200, 72), (5, 100000, 64)])
+def test_activation_in_the_products_epilogue_equals_the_two_kernels(kind, M, N, K):
+    from infinicore_infer_amd.kernels import ops
+    g = torch.Generator().manual_seed(M + N)
+    a = _dev(torch.randn(M, K, generator=g), torch.bfloat16)
+    w = _dev(torch.randn(N, K, generator=g) / math.sqrt(K), torch.bfloat16)
+    fused = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    plain = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    ops.gemm_nt(a, w, fused, activation=kind)
+    ops.gemm_nt(a, w, plain)
+    ops.activation(plain, plain, kind)
+    assert torch.equal(fused, plain)
