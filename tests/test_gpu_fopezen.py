@@ -469,3 +469,44 @@ def test_activation_in_the_products_epilogue_equals_the_two_kernels(kind, M, N, 
     ops.gemm_nt(a, w, plain)
     ops.activation(plain, plain, kind)
     assert torch.equal(fused, plain)
+
+
+@pytest.mark.parametrize("dname,dtype,tol", DTYPES)
+def test_forked_requests_go_on_independently(tmp_path_factory, dname, dtype, tol):
+    """A request's cache (planes of two widths, kept first pages, pages behind the window given back) copied into pages
+    of its own; the copy and the original go on with different tokens."""
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    folder, W = _model(tmp_path_factory, "F1")
+    eng = Engine.from_dir(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=4)
+    base = H.random_tokens(F1["vocab"], 97, 1)
+    tails = {"a": H.random_tokens(F1["vocab"], 30, 2), "b": H.random_tokens(F1["vocab"], 30, 3)}
+    eng.step([StepEntry("a", base[:60], [])])
+    eng.step([StepEntry("a", base[60:], [])])
+    eng.fork("a", "b")
+    eng.cache.check_invariants()
+    got = {}
+    for i in range(30):
+        rows = eng.step([StepEntry(r, [tails[r][i]], [0]) for r in ("a", "b")]).float().cpu()
+        for j, r in enumerate(("a", "b")):
+            got[(r, len(base) + i)] = rows[j].clone()
+    ref = {r: P.forward(F1, W, base + tails[r], torch.float64) for r in tails}
+    H.compare(got, ref, tol, "fork %s" % dname)
+    eng.free("a")
+    eng.free("b")
+    for g in range(len(eng.groups)):
+        assert eng.cache.free_pages(g) == eng.num_pages
+
+
+def test_command_line_with_random_weights(tmp_path):
+    """--random-weights --config: weights drawn for the configuration, several prompts through the scheduler."""
+    import subprocess
+    import sys
+    path = str(tmp_path / "config.json")
+    with open(path, "w") as f:
+        json.dump(F3, f)
+    r = subprocess.run([sys.executable, "-m", "infinicore_infer_amd.fopezen", "--amd", "--random-weights", "--config", path,
+                        "--prompt-len", "40", "--num-prompts", "3", "--max-new-tokens", "5", "--max-tokens", "256",
+                        "--max-batch-tokens", "64", "--chunk-size", "32", "--weights-norm-std", "0.05"],
+                       cwd=H.__file__.rsplit("/tests/", 1)[0], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert r.stdout.count("tokens[") == 3, r.stdout[-2000:]
