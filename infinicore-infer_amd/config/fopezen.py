@@ -106,8 +106,6 @@ class FopezenConfig:
     def validate(self) -> None:
         if self.vocab_size <= 0 or self.hidden_size <= 0:
             raise ConfigError("vocab and width must be positive")
-        if self.hidden_size % 2:
-            raise ConfigError("width (%d) must be even: the position vector pairs sines and cosines" % self.hidden_size)
         if not self.norm_eps > 0:
             raise ConfigError("norm.eps must be positive")
         if self.context_cap is not None and self.context_cap <= 0:

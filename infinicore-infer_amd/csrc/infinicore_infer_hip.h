@@ -66,7 +66,7 @@ int ic_attn_prefill_parts_of_step(int dtype, int n_tiles, int nh, int dh, int ma
 int ic_attn_prefill_split(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, int groups, int parts, int part_len, float* scratch, long long scratch_floats, int* counters, hipStream_t stream);
 
 // ---- stream_rows.hip: decoders whose sublayers read the residual stream and are normalised on the way back ----------
-// x[t, 2i] = table[tok, 2i] * scale + sin(p f_i), x[t, 2i+1] = .. + cos(p f_i) (freq: float32 [d/2]); copy (nullable): x in copy_dtype.
+// x[t, 2i] = table[tok, 2i] * scale + sin(p f_i), x[t, 2i+1] = .. + cos(p f_i) (freq: float32 [ceil(d/2)]); copy (nullable): x in copy_dtype.
 int ic_embed_sinusoid(const int* tokens, const int* positions, const void* table, int table_dtype, const float* freq, float* x, void* copy, int copy_dtype, int T, int d, float scale, hipStream_t stream);
 // x[t] += rmsnorm(y[t] + bias) * w (bias nullable, w float32 [d]); copy (nullable): the new x in copy_dtype.
 int ic_norm_into_stream(const void* y, int y_dtype, const float* bias, const float* w, float* x, void* copy, int copy_dtype, int T, int d, float eps, hipStream_t stream);

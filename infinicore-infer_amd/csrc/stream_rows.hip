@@ -41,7 +41,7 @@ template <> struct RowPack<bf16> {
 
 // ---------------------------------------------------------------------------------------------
 // x[t, 2i] = table[tok, 2i] * scale + sin(p f_i), x[t, 2i+1] = table[tok, 2i+1] * scale + cos(p f_i);
-// f_i is a float32 table [d/2] made by the host; the angle is the float32 product p * f_i.
+// f_i is a float32 table [ceil(d/2)] made by the host; the angle is the float32 product p * f_i.
 // copy (nullable): x rounded to the compute dtype.
 // ---------------------------------------------------------------------------------------------
 template <typename TW, typename TC>
@@ -52,15 +52,15 @@ __global__ void embed_sinusoid_kernel(const int* __restrict__ tokens, const int*
     const TW* row = table + (size_t)tokens[t] * d;
     const float p = (float)positions[t];
     float* o = x + (size_t)t * d;
-    for (int i = threadIdx.x; i < d / 2; i += blockDim.x) {
+    for (int i = threadIdx.x; i < (d + 1) / 2; i += blockDim.x) {
         const float ang = p * freq[i];
         const float a = to_f32(row[2 * i]) * scale + sinf(ang);
-        const float b = to_f32(row[2 * i + 1]) * scale + cosf(ang);
         o[2 * i] = a;
-        o[2 * i + 1] = b;
-        if (copy) {
-            copy[(size_t)t * d + 2 * i] = from_f32<TC>(a);
-            copy[(size_t)t * d + 2 * i + 1] = from_f32<TC>(b);
+        if (copy) copy[(size_t)t * d + 2 * i] = from_f32<TC>(a);
+        if (2 * i + 1 < d) {                              // an odd width ends on a sine
+            const float b = to_f32(row[2 * i + 1]) * scale + cosf(ang);
+            o[2 * i + 1] = b;
+            if (copy) copy[(size_t)t * d + 2 * i + 1] = from_f32<TC>(b);
         }
     }
 }
@@ -69,7 +69,7 @@ IC_EXPORT int ic_embed_sinusoid(const int* tokens, const int* positions, const v
                                 const float* freq, float* x, void* copy, int copy_dtype, int T, int d, float scale,
                                 hipStream_t stream) {
     if (T <= 0) return IC_OK;
-    if (d <= 0 || (d & 1)) return IC_ERR_ARG;
+    if (d <= 0) return IC_ERR_ARG;
     dim3 grid(T), block(256);
     if (table_dtype == IC_F32 && (copy == nullptr || copy_dtype == IC_F32))
         hipLaunchKernelGGL((embed_sinusoid_kernel<float, float>), grid, block, 0, stream, tokens, positions,

@@ -667,10 +667,10 @@ def embed_sinusoid(tokens, positions, table, freq, out, copy=None, scale: float 
     _i32(tokens, "tokens")
     _i32(positions, "positions")
     T, d = out.shape
-    _need(tokens.numel() == T and positions.numel() == T and table.dim() == 2 and table.shape[1] == d and d % 2 == 0,
+    _need(tokens.numel() == T and positions.numel() == T and table.dim() == 2 and table.shape[1] == d,
           "embed_sinusoid: shape mismatch")
     _need(out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous(), "embed_sinusoid: layout")
-    _need(freq.dtype == torch.float32 and freq.is_contiguous() and freq.numel() == d // 2, "embed_sinusoid: freq must be float32 [d/2]")
+    _need(freq.dtype == torch.float32 and freq.is_contiguous() and freq.numel() == (d + 1) // 2, "embed_sinusoid: freq must be float32 [ceil(d/2)]")
     if copy is not None:
         _need(tuple(copy.shape) == (T, d) and copy.is_contiguous(), "embed_sinusoid: copy layout")
     check(get_lib().ic_embed_sinusoid(tokens.data_ptr(), positions.data_ptr(), table.data_ptr(), dtype_code(table.dtype),

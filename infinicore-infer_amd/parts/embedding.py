@@ -17,9 +17,9 @@ from .linear import linear
 
 
 def sinusoid_frequencies(width: int, base: float) -> torch.Tensor:
-    """f_i = base^(-2i/width) for i < width/2, in float32 arithmetic (the angle of position p is the float32
+    """f_i = base^(-2i/width) for 2i < width, in float32 arithmetic (the angle of position p is the float32
     product p * f_i)."""
-    i = torch.arange(width // 2, dtype=torch.float32)
+    i = torch.arange((width + 1) // 2, dtype=torch.float32)
     return torch.pow(torch.tensor(base, dtype=torch.float32), -2.0 * i / width).contiguous()
 
 
@@ -32,7 +32,7 @@ class Embedding(Part):
     def __init__(self, name, runtime, vocab_size: int, hidden_size: int, scale: float = 1.0,
                  fallback_name=None, tensor=None, sinusoid_base=None):
         """``tensor``: the table's full name when it is not ``name + "weight"``.  ``sinusoid_base`` b: a position
-        vector is added to every row, entry 2i = sin(p b^(-2i/width)), entry 2i+1 = cos of the same angle."""
+        vector is added to every row, entry 2i = sin(p b^(-2i/width)), entry 2i+1 = cos of the same angle (an odd width ends on a sine)."""
         super().__init__(name, runtime)
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.scale = float(scale)
@@ -41,8 +41,6 @@ class Embedding(Part):
         self.table = None
         self.freq = None
         if sinusoid_base is not None:
-            if hidden_size % 2:
-                raise ValueError("a sinusoidal position vector needs an even width (got %d)" % hidden_size)
             self.freq = sinusoid_frequencies(hidden_size, float(sinusoid_base)).to(runtime.device)
         self.takes_context = self.freq is not None      # forward wants the step's positions
 

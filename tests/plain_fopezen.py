@@ -23,12 +23,12 @@ def norm_one_plus(x, w, eps):
 
 def sinusoid(positions, width, dtype):
     """Entry 2i is sin(p * 10000^(-2i/width)), entry 2i+1 the cosine of the same angle."""
-    i = torch.arange(width // 2, dtype=dtype)
+    i = torch.arange((width + 1) // 2, dtype=dtype)          # the arithmetic of the exponent is done in ``dtype``
     freq = torch.pow(torch.tensor(10000.0, dtype=dtype), -2.0 * i / width)
     ang = positions.to(dtype)[:, None] * freq[None, :]
     out = torch.zeros(len(positions), width, dtype=dtype)
     out[:, 0::2] = torch.sin(ang)
-    out[:, 1::2] = torch.cos(ang)
+    out[:, 1::2] = torch.cos(ang)[:, :width // 2]            # an odd width ends on a sine
     return out
 
 

@@ -36,7 +36,6 @@ def test_config_to_model_spec():
 @pytest.mark.parametrize("change,what", [
     (lambda c: c["layers"][0].update(type="attention_9"), "type"),
     (lambda c: c.pop("width"), "width"),
-    (lambda c: c.update(width=127), "even"),
     (lambda c: c["layers"][0]["mixer"].pop("scale"), "scale"),
     (lambda c: c["layers"][2]["mixer"].update(vdim=32), "agree"),
     (lambda c: c["layers"][0]["mixer"].update(heads=3), "multiple"),
