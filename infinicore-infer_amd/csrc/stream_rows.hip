@@ -207,8 +207,8 @@ qk_norm_store_kernel(const T* __restrict__ rows, int row_stride, const float* __
 
 // The same work 16 bytes a lane, for head sizes whose 16-byte pieces are a power of two per head (LPH lanes share a head of
 // q or k, LPV lanes a head of v) and rows that start on 16-byte boundaries.  Grid (tokens, ceil(items / 256)); an item is one
-// 16-byte piece of the row [q | k | v].  norm_mode 1: the lanes of a head sum their squares among themselves; norm_mode 2: every
-// wave sums the whole of q (or k) first.  A wave never straddles q/k and v pieces (the launcher pads the q/k pieces to whole waves).
+// 16-byte piece of the row [q | k | v].  norm_mode 0 or 1 (1: the lanes of a head sum their squares among themselves; the whole-row
+// norm has a kernel of its own below).  A wave never straddles q/k and v pieces (the launcher pads the q/k pieces to whole waves).
 template <typename T>
 __global__ void __launch_bounds__(256)
 qk_norm_store_vec_kernel(const T* __restrict__ rows, int row_stride, const float* __restrict__ bias,
@@ -244,23 +244,6 @@ qk_norm_store_vec_kernel(const T* __restrict__ rows, int row_stride, const float
             const float r = 1.0f / sqrtf(ss / (float)dk + eps);
 #pragma unroll
             for (int i = 0; i < N; ++i) val[i] = val[i] * r * w[j0 + i];
-        } else if (norm_mode == 2) {
-            // a wave's pieces may belong to q and to k: both sums are formed by every wave
-            float sq = 0.f, sk = 0.f;
-            for (int i = lane * N; i < nq + nk; i += 64 * N) {
-                float v[N];
-                RowPack<T>::load(src + i, v);
-                float s2 = 0.f;
-#pragma unroll
-                for (int e = 0; e < N; ++e) { const float z = v[e] + (bias ? bias[i + e] : 0.f); s2 += z * z; }
-                if (i < nq) sq += s2; else sk += s2;
-            }
-            sq = wave_sum(sq);
-            sk = wave_sum(sk);
-            const float r = is_q ? 1.0f / sqrtf(sq / (float)nq + eps) : 1.0f / sqrtf(sk / (float)nk + eps);
-            const int wj = is_q ? e0 : e0 - nq;
-#pragma unroll
-            for (int i = 0; i < N; ++i) val[i] = val[i] * r * w[wj + i];
         }
         if (!live) return;
         if (is_q) RowPack<T>::store(q_out + (size_t)t * nq + e0, val);
@@ -288,6 +271,66 @@ qk_norm_store_vec_kernel(const T* __restrict__ rows, int row_stride, const float
     (void)lpv;
 }
 
+// norm_mode 2, 16 bytes a lane: one block per token.  The sums of squares over the whole of q and of k are formed once
+// (first pass), then the row is read again (from cache), scaled and stored; the values follow.
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_store_whole_kernel(const T* __restrict__ rows, int row_stride, const float* __restrict__ bias,
+                           const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+                           int mix_mode, const float* __restrict__ lambda, float* __restrict__ v_keep,
+                           T* __restrict__ q_out, T* __restrict__ kcache, T* __restrict__ vcache,
+                           const int* __restrict__ slots, int nh, int nkvh, int dk, int dv, int page_size) {
+    constexpr int N = RowPack<T>::N;
+    __shared__ float red[16];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int nq = nh * dk, nk = nkvh * dk, nv = nkvh * dv;
+    const T* src = rows + (size_t)t * row_stride;
+    const int slot = slots ? slots[t] : -1;
+    const int pg = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - pg * page_size : 0;
+    const int qk_items = (nq + nk) / N;
+    float sq = 0.f, sk = 0.f;
+    for (int item = tid; item < qk_items; item += 256) {
+        float v[N];
+        RowPack<T>::load(src + item * N, v);
+        float s2 = 0.f;
+#pragma unroll
+        for (int e = 0; e < N; ++e) { const float z = v[e] + (bias ? bias[item * N + e] : 0.f); s2 += z * z; }
+        if (item * N < nq) sq += s2; else sk += s2;
+    }
+    sq = block_sum(sq, red);
+    sk = block_sum(sk, red);
+    const float rq = 1.0f / sqrtf(sq / (float)nq + eps), rk = 1.0f / sqrtf(sk / (float)nk + eps);
+    for (int item = tid; item < qk_items; item += 256) {
+        const int e0 = item * N;
+        const bool is_q = e0 < nq;
+        float v[N];
+        RowPack<T>::load(src + e0, v);
+        const float r = is_q ? rq : rk;
+        const float* w = is_q ? qw + e0 : kw + (e0 - nq);
+#pragma unroll
+        for (int e = 0; e < N; ++e) v[e] = (v[e] + (bias ? bias[e0 + e] : 0.f)) * r * w[e];
+        if (is_q) RowPack<T>::store(q_out + (size_t)t * nq + e0, v);
+        else if (slot >= 0 && kcache) {
+            const int kh = (e0 - nq) / dk, j0 = (e0 - nq) - kh * dk;
+            RowPack<T>::store(kcache + (((size_t)pg * nkvh + kh) * page_size + off) * dk + j0, v);
+        }
+    }
+    const float lam = (mix_mode == 2) ? lambda[0] : 0.f;
+    for (int vi = tid; vi < nv / N; vi += 256) {
+        const int e0 = vi * N, vh = e0 / dv, j0 = e0 - vh * dv;
+        float v[N];
+        RowPack<T>::load(src + nq + nk + e0, v);
+#pragma unroll
+        for (int e = 0; e < N; ++e) {
+            v[e] += bias ? bias[nq + nk + e0 + e] : 0.f;
+            float* keep = v_keep + (size_t)t * nv + e0 + e;
+            if (mix_mode == 1) *keep = v[e];
+            else if (mix_mode == 2) v[e] = (1.0f - lam) * v[e] + lam * *keep;
+        }
+        if (slot >= 0 && vcache) RowPack<T>::store(vcache + (((size_t)pg * nkvh + vh) * page_size + off) * dv + j0, v);
+    }
+}
+
 IC_EXPORT int ic_qk_norm_store(const void* rows, int row_stride, int dtype, const float* bias, const float* qw,
                                const float* kw, int norm_mode, float eps, int mix_mode, const float* lambda,
                                float* v_keep, void* q_out, void* kcache, void* vcache, const int* slots, int T, int nh,
@@ -311,6 +354,17 @@ IC_EXPORT int ic_qk_norm_store(const void* rows, int row_stride, int dtype, cons
         const bool pow2 = lph > 0 && lph <= 64 && (lph & (lph - 1)) == 0;
         const uintptr_t ptrs = (uintptr_t)rows | (uintptr_t)q_out | (uintptr_t)kcache | (uintptr_t)vcache;
         if ((dtype == IC_F32 || dtype == IC_BF16) && pow2 && dv % pack == 0 && row_stride % pack == 0 && (ptrs & 15) == 0) {
+            if (norm_mode == 2) {
+                if (dtype == IC_F32)
+                    hipLaunchKernelGGL(qk_norm_store_whole_kernel<float>, dim3(T), dim3(256), 0, stream, (const float*)rows, row_stride,
+                                       bias, qw, kw, eps, mix_mode, lambda, v_keep, (float*)q_out, (float*)kcache, (float*)vcache, slots,
+                                       nh, nkvh, dk, dv, page_size);
+                else
+                    hipLaunchKernelGGL(qk_norm_store_whole_kernel<bf16>, dim3(T), dim3(256), 0, stream, (const bf16*)rows, row_stride,
+                                       bias, qw, kw, eps, mix_mode, lambda, v_keep, (bf16*)q_out, (bf16*)kcache, (bf16*)vcache, slots, nh,
+                                       nkvh, dk, dv, page_size);
+                return ic_launch_status();
+            }
             const int qk_items = (int)(((long long)(nh + nkvh) * dk) / pack);
             const int qk_padded = (qk_items + 63) / 64 * 64;
             const int items = qk_padded + nkvh * dv / pack;
