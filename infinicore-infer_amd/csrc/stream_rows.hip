@@ -38,6 +38,14 @@ template <> struct RowPack<bf16> {
         *reinterpret_cast<v4u*>(p) = v;
     }
 };
+// N (4 or 8) float32 values from a 16-byte aligned address, 16 bytes a load.
+template <int N> __device__ __forceinline__ void load_floats(const float* p, float* o) {
+#pragma unroll
+    for (int i = 0; i < N / 4; ++i) {
+        const float4 v = *reinterpret_cast<const float4*>(p + 4 * i);
+        o[4 * i] = v.x; o[4 * i + 1] = v.y; o[4 * i + 2] = v.z; o[4 * i + 3] = v.w;
+    }
+}
 
 // ---------------------------------------------------------------------------------------------
 // x[t, 2i] = table[tok, 2i] * scale + sin(p f_i), x[t, 2i+1] = table[tok, 2i+1] * scale + cos(p f_i);
@@ -232,18 +240,21 @@ qk_norm_store_vec_kernel(const T* __restrict__ rows, int row_stride, const float
         const bool is_q = head < nh;
         RowPack<T>::load(src + e0, val);
         if (bias) {
+            float b[N];
+            load_floats<N>(bias + e0, b);
 #pragma unroll
-            for (int i = 0; i < N; ++i) val[i] += bias[e0 + i];
+            for (int i = 0; i < N; ++i) val[i] += b[i];
         }
-        const float* w = is_q ? qw : kw;
         if (norm_mode == 1) {
+            float wv[N];
+            load_floats<N>((is_q ? qw : kw) + j0, wv);
             float ss = 0.f;
 #pragma unroll
             for (int i = 0; i < N; ++i) ss += val[i] * val[i];
             for (int o = 1; o < lph; o <<= 1) ss += __shfl_xor(ss, o, kWave);       // lph is a power of two and divides 64
             const float r = 1.0f / sqrtf(ss / (float)dk + eps);
 #pragma unroll
-            for (int i = 0; i < N; ++i) val[i] = val[i] * r * w[j0 + i];
+            for (int i = 0; i < N; ++i) val[i] = val[i] * r * wv[i];
         }
         if (!live) return;
         if (is_q) RowPack<T>::store(q_out + (size_t)t * nq + e0, val);
@@ -256,25 +267,30 @@ qk_norm_store_vec_kernel(const T* __restrict__ rows, int row_stride, const float
     const int e0 = vi * N, vh = e0 / dv, j0 = e0 - vh * dv;
     RowPack<T>::load(src + nq + nk + e0, val);
     if (bias) {
+        float b[N];
+        load_floats<N>(bias + nq + nk + e0, b);
 #pragma unroll
-        for (int i = 0; i < N; ++i) val[i] += bias[nq + nk + e0 + i];
+        for (int i = 0; i < N; ++i) val[i] += b[i];
     }
+    float* keep = v_keep + (size_t)t * nv + e0;
     if (mix_mode == 1) {
 #pragma unroll
-        for (int i = 0; i < N; ++i) v_keep[(size_t)t * nv + e0 + i] = val[i];
+        for (int i = 0; i < N / 4; ++i) reinterpret_cast<float4*>(keep)[i] = make_float4(val[4 * i], val[4 * i + 1], val[4 * i + 2], val[4 * i + 3]);
     } else if (mix_mode == 2) {
         const float lam = lambda[0];
+        float kv[N];
+        load_floats<N>(keep, kv);
 #pragma unroll
-        for (int i = 0; i < N; ++i) val[i] = (1.0f - lam) * val[i] + lam * v_keep[(size_t)t * nv + e0 + i];
+        for (int i = 0; i < N; ++i) val[i] = (1.0f - lam) * val[i] + lam * kv[i];
     }
     if (slot >= 0 && vcache) RowPack<T>::store(vcache + (((size_t)pg * nkvh + vh) * page_size + off) * dv + j0, val);
     (void)lpv;
 }
 
-// norm_mode 2, 16 bytes a lane: one block per token.  The sums of squares over the whole of q and of k are formed once
+// norm_mode 2, 16 bytes a lane: one block per token (256 threads, or 1024 for rows of more than 512 pieces).  The sums of squares over the whole of q and of k are formed once
 // (first pass), then the row is read again (from cache), scaled and stored; the values follow.
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 qk_norm_store_whole_kernel(const T* __restrict__ rows, int row_stride, const float* __restrict__ bias,
                            const float* __restrict__ qw, const float* __restrict__ kw, float eps,
                            int mix_mode, const float* __restrict__ lambda, float* __restrict__ v_keep,
@@ -289,26 +305,28 @@ qk_norm_store_whole_kernel(const T* __restrict__ rows, int row_stride, const flo
     const int pg = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot - pg * page_size : 0;
     const int qk_items = (nq + nk) / N;
     float sq = 0.f, sk = 0.f;
-    for (int item = tid; item < qk_items; item += 256) {
-        float v[N];
+    for (int item = tid; item < qk_items; item += blockDim.x) {
+        float v[N], b[N];
         RowPack<T>::load(src + item * N, v);
+        if (bias) load_floats<N>(bias + item * N, b);
         float s2 = 0.f;
 #pragma unroll
-        for (int e = 0; e < N; ++e) { const float z = v[e] + (bias ? bias[item * N + e] : 0.f); s2 += z * z; }
+        for (int e = 0; e < N; ++e) { const float z = v[e] + (bias ? b[e] : 0.f); s2 += z * z; }
         if (item * N < nq) sq += s2; else sk += s2;
     }
     sq = block_sum(sq, red);
     sk = block_sum(sk, red);
     const float rq = 1.0f / sqrtf(sq / (float)nq + eps), rk = 1.0f / sqrtf(sk / (float)nk + eps);
-    for (int item = tid; item < qk_items; item += 256) {
+    for (int item = tid; item < qk_items; item += blockDim.x) {
         const int e0 = item * N;
         const bool is_q = e0 < nq;
-        float v[N];
+        float v[N], b[N], wv[N];
         RowPack<T>::load(src + e0, v);
+        if (bias) load_floats<N>(bias + e0, b);
+        load_floats<N>(is_q ? qw + e0 : kw + (e0 - nq), wv);
         const float r = is_q ? rq : rk;
-        const float* w = is_q ? qw + e0 : kw + (e0 - nq);
 #pragma unroll
-        for (int e = 0; e < N; ++e) v[e] = (v[e] + (bias ? bias[e0 + e] : 0.f)) * r * w[e];
+        for (int e = 0; e < N; ++e) v[e] = (v[e] + (bias ? b[e] : 0.f)) * r * wv[e];
         if (is_q) RowPack<T>::store(q_out + (size_t)t * nq + e0, v);
         else if (slot >= 0 && kcache) {
             const int kh = (e0 - nq) / dk, j0 = (e0 - nq) - kh * dk;
@@ -316,16 +334,21 @@ qk_norm_store_whole_kernel(const T* __restrict__ rows, int row_stride, const flo
         }
     }
     const float lam = (mix_mode == 2) ? lambda[0] : 0.f;
-    for (int vi = tid; vi < nv / N; vi += 256) {
+    for (int vi = tid; vi < nv / N; vi += blockDim.x) {
         const int e0 = vi * N, vh = e0 / dv, j0 = e0 - vh * dv;
-        float v[N];
+        float v[N], b[N], kv[N];
         RowPack<T>::load(src + nq + nk + e0, v);
+        if (bias) load_floats<N>(bias + nq + nk + e0, b);
+        float* keep = v_keep + (size_t)t * nv + e0;
+        if (mix_mode == 2) load_floats<N>(keep, kv);
 #pragma unroll
         for (int e = 0; e < N; ++e) {
-            v[e] += bias ? bias[nq + nk + e0 + e] : 0.f;
-            float* keep = v_keep + (size_t)t * nv + e0 + e;
-            if (mix_mode == 1) *keep = v[e];
-            else if (mix_mode == 2) v[e] = (1.0f - lam) * v[e] + lam * *keep;
+            v[e] += bias ? b[e] : 0.f;
+            if (mix_mode == 2) v[e] = (1.0f - lam) * v[e] + lam * kv[e];
+        }
+        if (mix_mode == 1) {
+#pragma unroll
+            for (int i = 0; i < N / 4; ++i) reinterpret_cast<float4*>(keep)[i] = make_float4(v[4 * i], v[4 * i + 1], v[4 * i + 2], v[4 * i + 3]);
         }
         if (slot >= 0 && vcache) RowPack<T>::store(vcache + (((size_t)pg * nkvh + vh) * page_size + off) * dv + j0, v);
     }
@@ -352,15 +375,17 @@ IC_EXPORT int ic_qk_norm_store(const void* rows, int row_stride, int dtype, cons
         const int pack = dtype == IC_F32 ? 4 : 8;
         const int lph = dk % pack == 0 ? dk / pack : 0;
         const bool pow2 = lph > 0 && lph <= 64 && (lph & (lph - 1)) == 0;
-        const uintptr_t ptrs = (uintptr_t)rows | (uintptr_t)q_out | (uintptr_t)kcache | (uintptr_t)vcache;
+        const uintptr_t ptrs = (uintptr_t)rows | (uintptr_t)q_out | (uintptr_t)kcache | (uintptr_t)vcache | (uintptr_t)bias |
+                               (uintptr_t)qw | (uintptr_t)kw | (uintptr_t)v_keep;
         if ((dtype == IC_F32 || dtype == IC_BF16) && pow2 && dv % pack == 0 && row_stride % pack == 0 && (ptrs & 15) == 0) {
             if (norm_mode == 2) {
+                const int threads = ((long long)(nh + nkvh) * dk / pack > 512) ? 1024 : 256;
                 if (dtype == IC_F32)
-                    hipLaunchKernelGGL(qk_norm_store_whole_kernel<float>, dim3(T), dim3(256), 0, stream, (const float*)rows, row_stride,
+                    hipLaunchKernelGGL(qk_norm_store_whole_kernel<float>, dim3(T), dim3(threads), 0, stream, (const float*)rows, row_stride,
                                        bias, qw, kw, eps, mix_mode, lambda, v_keep, (float*)q_out, (float*)kcache, (float*)vcache, slots,
                                        nh, nkvh, dk, dv, page_size);
                 else
-                    hipLaunchKernelGGL(qk_norm_store_whole_kernel<bf16>, dim3(T), dim3(256), 0, stream, (const bf16*)rows, row_stride,
+                    hipLaunchKernelGGL(qk_norm_store_whole_kernel<bf16>, dim3(T), dim3(threads), 0, stream, (const bf16*)rows, row_stride,
                                        bias, qw, kw, eps, mix_mode, lambda, v_keep, (bf16*)q_out, (bf16*)kcache, (bf16*)vcache, slots, nh,
                                        nkvh, dk, dv, page_size);
                 return ic_launch_status();

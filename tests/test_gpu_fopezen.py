@@ -339,7 +339,7 @@ def test_span_attention_kernels(case, dname, dtype, tol):
 @pytest.mark.parametrize("mode,mix", [(1, 0), (1, 1), (2, 2), (0, 2), (2, 0)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("Hq,G,dk,dv,extra", [(6, 3, 24, 40, 13), (4, 2, 64, 32, 16), (5, 5, 32, 128, 0), (3, 1, 128, 8, 24),
-                                              (4, 2, 64, 32, 3)])
+                                              (4, 2, 64, 32, 3), (40, 8, 128, 64, 0)])
 def test_bias_norm_value_mix_and_cache_write(mode, mix, dtype, Hq, G, dk, dv, extra):
     """Sizes that take the kernel's 16-byte path (pieces per head a power of two, aligned rows) and sizes that do not."""
     from infinicore_infer_amd.kernels import ops
