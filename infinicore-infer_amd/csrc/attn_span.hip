@@ -150,7 +150,7 @@ IC_EXPORT int ic_attn_span_generic(const void* q, int q_stride, void* out, int o
 //
 // Pass 1, grid (splits, kv heads, tokens), 256 threads: the visible keys of a token are numbered
 // 0 .. total-1 (the kept first keys, then the window); a block streams its share once and serves
-// every query head of the kv head, four at a time.  DK/VEC lanes share a key (VEC = 16 bytes of
+// every query head of the kv head, GQ (1, 2 or 4) at a time.  DK/VEC lanes share a key (VEC = 16 bytes of
 // elements), so a wave reads whole contiguous rows; the same lanes read the value row in pieces
 // of 16 bytes (a lane takes pieces sub, sub + LPK, .. when values are wider than keys, and none
 // when its piece lies beyond a narrower value row).  Every lane keeps a float32 running softmax
@@ -159,7 +159,6 @@ IC_EXPORT int ic_attn_span_generic(const void* q, int q_stride, void* out, int o
 // =============================================================================================
 constexpr int kSdThreads = 256;
 constexpr int kSdWaves = 4;
-constexpr int kSdGQ = 4;        // query heads served per walk over the keys
 constexpr int kSdUnroll = 4;    // keys a lane group has in flight
 constexpr float kLog2e = 1.4426950408889634f;
 
@@ -184,7 +183,7 @@ template <> struct SpanVec<bf16> {
 
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
-template <typename T, int DK, int DV>
+template <typename T, int DK, int DV, int GQ>
 __global__ void __launch_bounds__(kSdThreads)
 attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ kcache, const T* __restrict__ vcache,
                         const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_list,
@@ -199,8 +198,8 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
     constexpr int NVS = (LPV + LPK - 1) / LPK;     // value pieces per lane
     static_assert(DK % VEC == 0 && DV % VEC == 0 && 64 % LPK == 0 && LPK <= 64, "sizes must split a wave evenly");
 
-    __shared__ float sm_acc[kSdWaves][kSdGQ][DV];
-    __shared__ float sm_ml[kSdWaves][kSdGQ][2];
+    __shared__ float sm_acc[kSdWaves][GQ][DV];
+    __shared__ float sm_ml[kSdWaves][GQ][2];
 
     const int split = blockIdx.x, kvh = blockIdx.y, n = blockIdx.z;
     const int t = tok_list ? tok_list[n] : n;
@@ -217,10 +216,10 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
     const int sub = lane % LPK, grp = lane / LPK;
     const float qscale = scale * kLog2e;           // scores in units of log 2
 
-    for (int h0 = 0; h0 < g; h0 += kSdGQ) {
-        float qv[kSdGQ][VEC], acc[kSdGQ][NVS * VEC], m[kSdGQ], l[kSdGQ];
+    for (int h0 = 0; h0 < g; h0 += GQ) {
+        float qv[GQ][VEC], acc[GQ][NVS * VEC], m[GQ], l[GQ];
 #pragma unroll
-        for (int j = 0; j < kSdGQ; ++j) {
+        for (int j = 0; j < GQ; ++j) {
             m[j] = -INFINITY; l[j] = 0.f;
             const int hh = (h0 + j < g) ? h0 + j : g - 1;
             SpanVec<T>::load(q + (size_t)t * q_stride + (size_t)(kvh * g + hh) * DK + sub * VEC, qv[j]);
@@ -261,7 +260,7 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
             }
             if (ib + STEP - grp - wave * KPW < hi) look(ib + STEP);
 #pragma unroll
-            for (int j = 0; j < kSdGQ; ++j) {
+            for (int j = 0; j < GQ; ++j) {
                 float s[kSdUnroll];
                 float mx = m[j];
 #pragma unroll
@@ -269,8 +268,7 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
                     float d = 0.f;
 #pragma unroll
                     for (int i = 0; i < VEC; ++i) d += qv[j][i] * kf[u][i];
-#pragma unroll
-                    for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, kWave);
+                    d = group_sum<LPK>(d);                  // over the lanes that share the key (DPP steps inside a row of 16 lanes)
                     s[u] = ok[u] ? d : -INFINITY;
                     mx = fmaxf(mx, s[u]);
                 }
@@ -292,7 +290,7 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
         }
         // merge the lane groups of the wave (lanes with the same `sub`)
 #pragma unroll
-        for (int j = 0; j < kSdGQ; ++j) {
+        for (int j = 0; j < GQ; ++j) {
 #pragma unroll
             for (int o = LPK; o < 64; o <<= 1) {
                 const float mb = __shfl_xor(m[j], o, kWave);
@@ -309,7 +307,7 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
         __syncthreads();                                // LDS free from the previous chunk of heads
         if (grp == 0) {
 #pragma unroll
-            for (int j = 0; j < kSdGQ; ++j) {
+            for (int j = 0; j < GQ; ++j) {
 #pragma unroll
                 for (int s = 0; s < NVS; ++s)
                     if (sub + s * LPK < LPV)
@@ -319,7 +317,7 @@ attn_span_decode_kernel(const T* __restrict__ q, int q_stride, const T* __restri
             }
         }
         __syncthreads();
-        for (int idx = threadIdx.x; idx < kSdGQ * DV; idx += kSdThreads) {
+        for (int idx = threadIdx.x; idx < GQ * DV; idx += kSdThreads) {
             const int j = idx / DV, d = idx - j * DV;
             if (h0 + j >= g) continue;
             float mm = -INFINITY;
@@ -402,10 +400,16 @@ static int span_decode_launch(const void* q, int q_stride, void* out, int out_st
                               float* part_ml, int n_tok, int nh, int nkvh, int page_size, float scale, int window,
                               int keep_first, int sink, int nsplit, hipStream_t stream) {
     dim3 grid(nsplit, nkvh, n_tok), block(kSdThreads);
-    hipLaunchKernelGGL((attn_span_decode_kernel<T, DK, DV>), grid, block, 0, stream, (const T*)q, q_stride, (const T*)kcache,
-                       (const T*)vcache, block_tables, bt_stride, tok_list, token_req, positions, part_acc, part_ml, nh, nkvh,
-                       page_size, scale, window, keep_first, nsplit, sink, nsplit == 1 ? (T*)out : (T*)nullptr, out_stride,
-                       (const T*)gate, gate_stride);
+    const int g = nh / nkvh;
+#define IC_SPAN_GQ(GQ)                                                                                                          \
+    hipLaunchKernelGGL((attn_span_decode_kernel<T, DK, DV, GQ>), grid, block, 0, stream, (const T*)q, q_stride, (const T*)kcache, \
+                       (const T*)vcache, block_tables, bt_stride, tok_list, token_req, positions, part_acc, part_ml, nh, nkvh,   \
+                       page_size, scale, window, keep_first, nsplit, sink, nsplit == 1 ? (T*)out : (T*)nullptr, out_stride,     \
+                       (const T*)gate, gate_stride)
+    if (g == 1) IC_SPAN_GQ(1);                      // query heads served per walk over the keys: no more than there are
+    else if (g == 2) IC_SPAN_GQ(2);
+    else IC_SPAN_GQ(4);
+#undef IC_SPAN_GQ
     int st = ic_launch_status();
     if (st != IC_OK || nsplit == 1) return st;
     hipLaunchKernelGGL(attn_span_reduce_kernel<T>, dim3((unsigned)(n_tok * nh)), dim3(DV < 64 ? 64 : DV), 0, stream, part_acc,

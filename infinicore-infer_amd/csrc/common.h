@@ -69,6 +69,22 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Sum over the LPK consecutive lanes that share a key; every one of them gets the same total.
+// Steps inside a row of 16 lanes are DPP operands of the add (no LDS round trip).
+__device__ __forceinline__ float dpp_add(float v, int) = delete;
+template <int CTRL> __device__ __forceinline__ float dpp_add(float v) {
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int LPK> __device__ __forceinline__ float group_sum(float d) {
+    if (LPK >= 64) d += __shfl_xor(d, 32, kWave);
+    if (LPK >= 32) d += __shfl_xor(d, 16, kWave);
+    if (LPK >= 16) d = dpp_add<0x128>(d);        // row_ror:8      lane i <- lane i ^ 8
+    if (LPK >= 8) d = dpp_add<0x141>(d);         // row_half_mirror lane i <- lane 7 - i (of 8)
+    if (LPK >= 4) d = dpp_add<0x4E>(d);          // quad_perm [2,3,0,1]
+    if (LPK >= 2) d = dpp_add<0xB1>(d);          // quad_perm [1,0,3,2]
+    return d;
+}
+
 // Sum over a whole block; every thread gets the result.  `red` is LDS of at
 // least blockDim.x / 64 floats.  Safe to call repeatedly with the same `red`.
 __device__ __forceinline__ float block_sum(float v, float* red) {
