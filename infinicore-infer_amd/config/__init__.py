@@ -4,10 +4,11 @@ from .registry import (ConfigError, config_from_dict, config_from_dir, read_conf
 from .spec import ExecEntry, LayerSpec, ModelSpec, PartSpec, default_schedule
 from .minicpm import MiniCPMConfig, RopeScaling
 from .fopezen import FopezenConfig
+from .mezinex import MezinexConfig
 
 __all__ = [
     "ConfigError", "config_from_dict", "config_from_dir", "read_config_json",
     "register_architecture", "registered_architectures", "resolve_architecture",
     "ExecEntry", "LayerSpec", "ModelSpec", "PartSpec", "default_schedule",
-    "MiniCPMConfig", "RopeScaling", "FopezenConfig",
+    "MiniCPMConfig", "RopeScaling", "FopezenConfig", "MezinexConfig",
 ]

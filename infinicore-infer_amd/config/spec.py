@@ -62,6 +62,7 @@ class ModelSpec:
     head: PartSpec
     eos_token_ids: List[int] = field(default_factory=list)
     bos_token_id: Optional[int] = None
+    residual_streams: int = 1          # float32 copies of the residual stream that the blocks keep ([S, T, d] when > 1)
 
     def num_cache_slots(self) -> int:
         return 1 + max((e.cache for e in self.schedule), default=-1)

@@ -1,0 +1,344 @@
+// Mixers that carry a fixed-size state per sequence instead of a cache of keys: a short causal convolution
+// per channel, a gated diagonal linear recurrence, a state-space recurrence with a matrix state per head, the
+// gated norm in groups that follows it, and a product with one small weight matrix per block of columns.
+//
+// A step's tokens are rows 0..T-1; request r owns rows req_start[r] .. req_start[r+1]-1 and the state slot
+// state_slots[r].  State lives in float32, [slots, state_stride] floats, a part of a mixer's state at an offset.
+// Everything that enters a recurrence is float32.
+#include "common.h"
+
+constexpr int kConvMaxTaps = 8;
+
+__device__ __forceinline__ float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// ---- causal convolution per channel -----------------------------------------------------------------------
+// in(t, c) = xin[t, c] + in_bias[c]; out(t, c) = act(b[c] + sum_k w[c, k] in(t - (taps-1-k), c)); inputs before
+// the step's first row come from the state (the last taps-1 inputs, oldest first), zeros for a new sequence.
+template <typename T>
+__global__ void __launch_bounds__(256)
+causal_conv_kernel(const T* __restrict__ xin, int xin_stride, const float* __restrict__ in_bias,
+                   const float* __restrict__ w, const float* __restrict__ b, int taps, int C,
+                   float* __restrict__ out, T* __restrict__ out_copy, int copy_stride, int act,
+                   const float* __restrict__ state, long long state_stride,
+                   const int* __restrict__ token_req, const int* __restrict__ req_start,
+                   const int* __restrict__ state_slots) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, t = blockIdx.y;
+    if (c >= C) return;
+    const int r = token_req[t];
+    const int start = req_start[r];
+    const float* st = state + (long long)state_slots[r] * state_stride;
+    const float ib = in_bias ? in_bias[c] : 0.f;
+    float acc = b ? b[c] : 0.f;
+    for (int k = 0; k < taps; ++k) {
+        const int src = t - (taps - 1 - k);
+        float v;
+        if (src >= start) v = to_f32(xin[(size_t)src * xin_stride + c]) + ib;
+        else v = st[(size_t)(taps - 1 - (start - src)) * C + c];
+        acc += w[(size_t)c * taps + k] * v;
+    }
+    if (act == 1) acc = silu_f(acc);
+    out[(size_t)t * C + c] = acc;
+    if (out_copy) out_copy[(size_t)t * copy_stride + c] = from_f32<T>(acc);
+}
+
+// The state after the step: the last taps-1 of (old state, the step's inputs).  One thread per (request, channel).
+template <typename T>
+__global__ void __launch_bounds__(256)
+conv_state_kernel(const T* __restrict__ xin, int xin_stride, const float* __restrict__ in_bias, int taps, int C,
+                  float* __restrict__ state, long long state_stride, const int* __restrict__ req_start,
+                  const int* __restrict__ state_slots) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+    if (c >= C) return;
+    const int start = req_start[r], n = req_start[r + 1] - start;
+    float* st = state + (long long)state_slots[r] * state_stride;
+    const float ib = in_bias ? in_bias[c] : 0.f;
+    float nv[kConvMaxTaps];
+    for (int k = 0; k < taps - 1; ++k) {
+        const int i = n + k;                      // index into (old state, inputs)
+        nv[k] = i < taps - 1 ? st[(size_t)i * C + c]
+                             : to_f32(xin[(size_t)(start + i - (taps - 1)) * xin_stride + c]) + ib;
+    }
+    for (int k = 0; k < taps - 1; ++k) st[(size_t)k * C + c] = nv[k];
+}
+
+IC_EXPORT int ic_causal_conv(const void* xin, int xin_stride, int dtype, const float* in_bias, const float* w,
+                             const float* b, int taps, int C, float* out, void* out_copy, int copy_stride, int act,
+                             float* state, long long state_stride, const int* token_req, const int* req_start,
+                             const int* state_slots, int T, int R, hipStream_t stream) {
+    if (T <= 0) return IC_OK;
+    if (taps < 1 || taps > kConvMaxTaps || C <= 0 || R <= 0 || !state || !req_start || !state_slots) return IC_ERR_ARG;
+    dim3 grid((C + 255) / 256, T), sgrid((C + 255) / 256, R), block(256);
+    if (dtype == IC_F32) {
+        hipLaunchKernelGGL(causal_conv_kernel<float>, grid, block, 0, stream, (const float*)xin, xin_stride, in_bias, w, b,
+                           taps, C, out, (float*)out_copy, copy_stride, act, state, state_stride, token_req, req_start,
+                           state_slots);
+        if (taps > 1)
+            hipLaunchKernelGGL(conv_state_kernel<float>, sgrid, block, 0, stream, (const float*)xin, xin_stride, in_bias,
+                               taps, C, state, state_stride, req_start, state_slots);
+    } else if (dtype == IC_BF16) {
+        hipLaunchKernelGGL(causal_conv_kernel<bf16>, grid, block, 0, stream, (const bf16*)xin, xin_stride, in_bias, w, b,
+                           taps, C, out, (bf16*)out_copy, copy_stride, act, state, state_stride, token_req, req_start,
+                           state_slots);
+        if (taps > 1)
+            hipLaunchKernelGGL(conv_state_kernel<bf16>, sgrid, block, 0, stream, (const bf16*)xin, xin_stride, in_bias,
+                               taps, C, state, state_stride, req_start, state_slots);
+    } else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// ---- gated diagonal linear recurrence -------------------------------------------------------------------------
+// Channel c lies in block c / bw; its gate pre-activations are gates[t, (c / bw) * 2 bw + c % bw] (recurrence
+// gate) and the same + bw (input gate), biases laid out alike.  With r, i their sigmoids:
+//     log a = decay[c] * r,  S <- exp(log a) S + sqrt(1 - exp(2 log a)) * i * u,  out = S * gelu_tanh(yb + y_bias).
+// decay[c] = -8 softplus(lam[c]), made once when the weights are loaded.
+template <typename T>
+__global__ void __launch_bounds__(128)
+rglru_scan_kernel(const float* __restrict__ gates, const float* __restrict__ gate_bias, const float* __restrict__ u,
+                  const T* __restrict__ yb, int yb_stride, const float* __restrict__ y_bias,
+                  const float* __restrict__ decay, int width, int bw, T* __restrict__ out,
+                  float* __restrict__ state, long long state_stride, const int* __restrict__ req_start,
+                  const int* __restrict__ state_slots) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+    if (c >= width) return;
+    const int g0 = (c / bw) * 2 * bw + c % bw;
+    const float br = gate_bias[g0], bi = gate_bias[g0 + bw], dc = decay[c], yb0 = y_bias ? y_bias[c] : 0.f;
+    float* st = state + (long long)state_slots[r] * state_stride;
+    float S = st[c];
+    const int end = req_start[r + 1];
+    for (int t = req_start[r]; t < end; ++t) {
+        const float* g = gates + (size_t)t * 2 * width;
+        const float rg = sigmoid_f(g[g0] + br), ig = sigmoid_f(g[g0 + bw] + bi);
+        const float la = dc * rg;
+        S = expf(la) * S + sqrtf(-expm1f(2.0f * la)) * ig * u[(size_t)t * width + c];
+        out[(size_t)t * width + c] = from_f32<T>(S * gelu_tanh_f(to_f32(yb[(size_t)t * yb_stride + c]) + yb0));
+    }
+    st[c] = S;
+}
+
+IC_EXPORT int ic_rglru_scan(const float* gates, const float* gate_bias, const float* u, const void* yb, int yb_stride,
+                            int dtype, const float* y_bias, const float* decay, int width, int bw, void* out,
+                            float* state, long long state_stride, const int* req_start, const int* state_slots, int R,
+                            hipStream_t stream) {
+    if (R <= 0) return IC_OK;
+    if (width <= 0 || bw <= 0 || width % bw || !state) return IC_ERR_ARG;
+    dim3 grid((width + 127) / 128, R), block(128);
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(rglru_scan_kernel<float>, grid, block, 0, stream, gates, gate_bias, u, (const float*)yb, yb_stride,
+                           y_bias, decay, width, bw, (float*)out, state, state_stride, req_start, state_slots);
+    else if (dtype == IC_BF16)
+        hipLaunchKernelGGL(rglru_scan_kernel<bf16>, grid, block, 0, stream, gates, gate_bias, u, (const bf16*)yb, yb_stride,
+                           y_bias, decay, width, bw, (bf16*)out, state, state_stride, req_start, state_slots);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// ---- state-space recurrence with a matrix state per head ---------------------------------------------------------
+// xbc [T, inner + 2 G N] float32 holds x (heads x P), then B (G x N), then C (G x N) of every token.  Per head h
+// with group g = h / (heads / G), dt = softplus(dt_raw + dt_bias[h]):
+//     S <- exp(neg_a[h] dt) S + dt B_g x_h^T   (S is N x P),   y_h = S^T C_g + D[h] x_h.
+// One block per (head, request); the state stays in LDS while the block walks the request's tokens.
+template <typename T>
+__global__ void __launch_bounds__(256)
+ssm_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ dt_raw, int dt_stride,
+                const float* __restrict__ dt_bias, const float* __restrict__ neg_a, const float* __restrict__ Dw,
+                int heads, int P, int N, int G, float* __restrict__ y, float* __restrict__ state,
+                long long state_stride, const int* __restrict__ req_start, const int* __restrict__ state_slots) {
+    extern __shared__ float lds[];
+    const int h = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+    const int g = h / (heads / G), inner = heads * P, ch = inner + 2 * G * N;
+    const int ngrp = 256 / P;                    // P <= 256
+    float* S = lds;                              // N * P
+    float* Bs = S + (size_t)N * P;               // N
+    float* Cs = Bs + N;                          // N
+    float* xs = Cs + N;                          // P
+    float* part = xs + P;                        // ngrp * P
+    float* st = state + (long long)state_slots[r] * state_stride + (size_t)h * N * P;
+    for (int e = tid; e < N * P; e += 256) S[e] = st[e];
+    const float db = dt_bias[h], na = neg_a[h], dw = Dw[h];
+    const int grp = tid / P, p = tid % P;
+    const int end = req_start[r + 1];
+    __syncthreads();
+    for (int t = req_start[r]; t < end; ++t) {
+        const float* row = xbc + (size_t)t * ch;
+        for (int n = tid; n < N; n += 256) {
+            Bs[n] = row[inner + g * N + n];
+            Cs[n] = row[inner + G * N + g * N + n];
+        }
+        for (int q = tid; q < P; q += 256) xs[q] = row[h * P + q];
+        const float dt = softplus_f(to_f32(dt_raw[(size_t)t * dt_stride + h]) + db);
+        const float da = expf(na * dt);
+        __syncthreads();
+        if (grp < ngrp) {
+            const float dx = dt * xs[p];
+            float acc = 0.f;
+            for (int n = grp; n < N; n += ngrp) {
+                const float s = da * S[n * P + p] + Bs[n] * dx;
+                S[n * P + p] = s;
+                acc += s * Cs[n];
+            }
+            part[grp * P + p] = acc;
+        }
+        __syncthreads();
+        if (tid < P) {
+            float acc = dw * xs[tid];
+            for (int q = 0; q < ngrp; ++q) acc += part[q * P + tid];
+            y[(size_t)t * inner + h * P + tid] = acc;
+        }
+        __syncthreads();
+    }
+    for (int e = tid; e < N * P; e += 256) st[e] = S[e];
+}
+
+IC_EXPORT int ic_ssm_scan(const float* xbc, const void* dt_raw, int dt_stride, int dtype, const float* dt_bias,
+                          const float* neg_a, const float* Dw, int heads, int P, int N, int G, float* y, float* state,
+                          long long state_stride, const int* req_start, const int* state_slots, int R,
+                          hipStream_t stream) {
+    if (R <= 0) return IC_OK;
+    if (heads <= 0 || P <= 0 || P > 256 || N <= 0 || G <= 0 || heads % G || !state) return IC_ERR_ARG;
+    const size_t lds = ((size_t)N * P + 2 * N + P + (size_t)(256 / P) * P) * sizeof(float);
+    if (lds > 64 * 1024) return IC_ERR_TOO_LARGE;
+    dim3 grid(heads, R), block(256);
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(ssm_scan_kernel<float>, grid, block, lds, stream, xbc, (const float*)dt_raw, dt_stride, dt_bias,
+                           neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots);
+    else if (dtype == IC_BF16)
+        hipLaunchKernelGGL(ssm_scan_kernel<bf16>, grid, block, lds, stream, xbc, (const bf16*)dt_raw, dt_stride, dt_bias,
+                           neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// ---- gate, then RMS norm in groups ----------------------------------------------------------------------------------
+// v = y * silu(z); every group of `gs` columns is divided by its own root mean square; times w.  One block per
+// (token, group).
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, int z_stride, const float* __restrict__ w,
+                        int inner, int gs, float eps, T* __restrict__ out) {
+    extern __shared__ float v_row[];          // gs floats
+    __shared__ float red[8];
+    const int t = blockIdx.x, c0 = blockIdx.y * gs;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < gs; j += blockDim.x) {
+        const float v = y[(size_t)t * inner + c0 + j] * silu_f(to_f32(z[(size_t)t * z_stride + c0 + j]));
+        v_row[j] = v;
+        ss += v * v;
+    }
+    const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)gs + eps);
+    for (int j = threadIdx.x; j < gs; j += blockDim.x)
+        out[(size_t)t * inner + c0 + j] = from_f32<T>(v_row[j] * r * w[c0 + j]);
+}
+
+IC_EXPORT int ic_gated_group_norm(const float* y, const void* z, int z_stride, int dtype, const float* w, int inner,
+                                  int groups, float eps, void* out, int T, hipStream_t stream) {
+    if (T <= 0) return IC_OK;
+    if (inner <= 0 || groups <= 0 || inner % groups || inner / groups > 16384) return IC_ERR_ARG;
+    const int gs = inner / groups;
+    dim3 grid(T, groups), block(256);
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(gated_group_norm_kernel<float>, grid, block, gs * sizeof(float), stream, y, (const float*)z,
+                           z_stride, w, inner, gs, eps, (float*)out);
+    else if (dtype == IC_BF16)
+        hipLaunchKernelGGL(gated_group_norm_kernel<bf16>, grid, block, gs * sizeof(float), stream, y, (const bf16*)z,
+                           z_stride, w, inner, gs, eps, (bf16*)out);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// ---- a product with one weight matrix per block of columns --------------------------------------------------------------
+// C[m, b * c_step + n] = sum_k A[m, b * a_step + k] W[b, n, k]  (b < B, n < N, k < K; W contiguous [B, N, K]),
+// optionally times sigmoid(gate[m, b * c_step + n]).  float32 accumulation on the vector units; tiles of BM x 64
+// results per block of 256 threads, 16 k at a time through LDS.
+template <typename T, typename TC, int BM>
+__global__ void __launch_bounds__(256)
+blocked_product_kernel(const T* __restrict__ A, int lda, int a_step, const T* __restrict__ W, TC* __restrict__ C,
+                       int ldc, int c_step, const T* __restrict__ gate, int gate_stride, int M, int N, int K) {
+    constexpr int BN = 64, BK = 16, RM = BM / 16;
+    __shared__ float As[BK][BM + 1];
+    __shared__ float Ws[BK][BN + 1];
+    const int b = blockIdx.z, m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const T* Ab = A + (size_t)b * a_step;
+    const T* Wb = W + (size_t)b * N * K;
+    float acc[RM][4];
+#pragma unroll
+    for (int i = 0; i < RM; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        for (int e = threadIdx.x; e < BM * BK; e += 256) {
+            const int m = e / BK, k = e % BK;
+            As[k][m] = (m0 + m < M && k0 + k < K) ? to_f32(Ab[(size_t)(m0 + m) * lda + k0 + k]) : 0.f;
+        }
+        for (int e = threadIdx.x; e < BN * BK; e += 256) {
+            const int n = e / BK, k = e % BK;
+            Ws[k][n] = (n0 + n < N && k0 + k < K) ? to_f32(Wb[(size_t)(n0 + n) * K + k0 + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; ++k) {
+            float a[RM], w[4];
+#pragma unroll
+            for (int i = 0; i < RM; ++i) a[i] = As[k][ty * RM + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = Ws[k][tx + 16 * j];
+#pragma unroll
+            for (int i = 0; i < RM; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * w[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < RM; ++i) {
+        const int m = m0 + ty * RM + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx + 16 * j;
+            if (n >= N) continue;
+            float v = acc[i][j];
+            if (gate) v *= sigmoid_f(to_f32(gate[(size_t)m * gate_stride + (size_t)b * c_step + n]));
+            C[(size_t)m * ldc + (size_t)b * c_step + n] = from_f32<TC>(v);
+        }
+    }
+}
+
+template <typename T, typename TC>
+static void blocked_product_launch(const void* A, int lda, int a_step, const void* W, void* C, int ldc, int c_step,
+                                   const void* gate, int gate_stride, int M, int N, int K, int B, hipStream_t stream) {
+    if (M <= 16) {
+        dim3 grid((N + 63) / 64, (M + 15) / 16, B);
+        hipLaunchKernelGGL((blocked_product_kernel<T, TC, 16>), grid, dim3(256), 0, stream, (const T*)A, lda, a_step,
+                           (const T*)W, (TC*)C, ldc, c_step, (const T*)gate, gate_stride, M, N, K);
+    } else {
+        dim3 grid((N + 63) / 64, (M + 63) / 64, B);
+        hipLaunchKernelGGL((blocked_product_kernel<T, TC, 64>), grid, dim3(256), 0, stream, (const T*)A, lda, a_step,
+                           (const T*)W, (TC*)C, ldc, c_step, (const T*)gate, gate_stride, M, N, K);
+    }
+}
+
+IC_EXPORT int ic_blocked_product(const void* A, int lda, int a_step, const void* W, int dtype, void* C, int c_dtype,
+                                 int ldc, int c_step, const void* gate, int gate_stride, int M, int N, int K, int B,
+                                 hipStream_t stream) {
+    if (M <= 0) return IC_OK;
+    if (N <= 0 || K <= 0 || B <= 0 || B > 65535 || (M + 15) / 16 > 65535) return IC_ERR_ARG;
+    if (dtype == IC_F32 && c_dtype == IC_F32)
+        blocked_product_launch<float, float>(A, lda, a_step, W, C, ldc, c_step, gate, gate_stride, M, N, K, B, stream);
+    else if (dtype == IC_BF16 && c_dtype == IC_BF16)
+        blocked_product_launch<bf16, bf16>(A, lda, a_step, W, C, ldc, c_step, gate, gate_stride, M, N, K, B, stream);
+    else if (dtype == IC_BF16 && c_dtype == IC_F32)
+        blocked_product_launch<bf16, float>(A, lda, a_step, W, C, ldc, c_step, gate, gate_stride, M, N, K, B, stream);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}

@@ -92,6 +92,9 @@ class StepContext:
         self.positions = None            # int32 [T]
         self.token_req = None            # int32 [T]  batch row of each token
         self.state_slots = None          # int32 [R]  state slot of each request
+        self.req_rows = None             # int32 [R + 1]  first token row of each request, then T
+        self.embedding_state = None      # [max_requests, ...] what the embedding keeps per request, if anything
+        self.layer_probe = None          # tests: called as probe(entry index, x, pending) after every entry of the run order
         self.want_rows = None            # int32 [W]  token rows whose logits are wanted
         self.n_want = 0
         self.want_rows_identity = False  # every row's logits are wanted, in order

@@ -111,6 +111,9 @@ class Engine:
         for slot, need in enumerate(needs):
             if need.has_state:
                 self.storage.add_state(slot, self.max_requests, need.state_shape, need.state_dtype)
+        emb_need = model.embedding_cache_need() if hasattr(model, "embedding_cache_need") else None
+        if emb_need is not None and emb_need.has_state:      # what the embedding keeps per request lives with the mixers' states
+            self.storage.add_state("embedding", self.max_requests, emb_need.state_shape, emb_need.state_dtype)
         self._slot_group = {s: g for g, spec in enumerate(self.groups) for s in spec.slots}
         self.has_state = bool(self.storage.state)      # some mixer keeps fixed-size state per request
         self._has_window = any(g.kind == "window" for g in self.groups)
@@ -441,7 +444,7 @@ class Engine:
         n_groups = len(self.groups)
         tables = [[self.cache.block_table(e.req_id, g) for e in entries] for g in range(n_groups)]
         group_maxb = [max([1] + [len(t) for t in tables[g]]) for g in range(n_groups)]
-        sizes = [("tokens", T), ("positions", T), ("token_req", T), ("state_slots", R),
+        sizes = [("tokens", T), ("positions", T), ("token_req", T), ("state_slots", R), ("req_rows", R + 1),
                  ("want_rows", len(want_rows)), ("decode_rows", len(decode_rows)), ("tiles", 4 * len(tiles))]
         for g in range(n_groups):
             sizes += [("slots%d" % g, T), ("tables%d" % g, R * group_maxb[g])]
@@ -473,6 +476,7 @@ class Engine:
                 a[o:o + len(table)] = np.maximum(table, 0)     # pages given back are never read; keep the index valid
                 a[o + len(table):o + group_maxb[g]] = 0
         put("state_slots", state_slots)
+        put("req_rows", req_start)
         put("want_rows", want_rows)
         put("decode_rows", decode_rows)
         if tiles:
@@ -490,7 +494,8 @@ class Engine:
         ctx = StepContext()
         ctx.T, ctx.R, ctx.page_size, ctx.ws = T, R, ps, self.ws
         ctx.tokens, ctx.positions, ctx.token_req = view("tokens"), view("positions"), view("token_req")
-        ctx.state_slots = view("state_slots")
+        ctx.state_slots, ctx.req_rows = view("state_slots"), view("req_rows")
+        ctx.embedding_state = self.storage.state.get("embedding")
         ctx.want_rows, ctx.n_want = view("want_rows"), len(want_rows)
         ctx.want_rows_identity = (len(want_rows) == T and all(w == i for i, w in enumerate(want_rows)))
         ctx.decode_rows, ctx.n_decode_rows = view("decode_rows"), len(decode_rows)
@@ -695,8 +700,9 @@ class _DecodeGraph:
         self.R = R
         ng = len(engine.groups)
         self.maxb = (engine.model.spec.max_positions + engine.page_size - 1) // engine.page_size
-        names = ["tokens", "positions", "token_req", "state_slots", "want_rows"]
+        names = ["tokens", "positions", "token_req", "state_slots", "want_rows", "req_rows"]
         sizes = {n: R for n in names}
+        sizes["req_rows"] = R + 1
         for g in range(ng):
             names += ["slots%d" % g, "tables%d" % g]
             sizes["slots%d" % g] = R
@@ -715,6 +721,7 @@ class _DecodeGraph:
         self.copied.record()
         self.np[self.off["token_req"]:self.off["token_req"] + R] = range(R)
         self.np[self.off["want_rows"]:self.off["want_rows"] + R] = range(R)
+        self.np[self.off["req_rows"]:self.off["req_rows"] + R + 1] = range(R + 1)
         self._row_keys = [[None] * R for _ in range(ng)]
         self.graph = None
         self.logits = None
@@ -726,7 +733,8 @@ class _DecodeGraph:
         # the recorded launches hold the workspace's addresses, so it must never be regrown
         ctx.T, ctx.R, ctx.page_size, ctx.ws = R, R, engine.page_size, engine._graph_workspace()
         ctx.tokens, ctx.positions, ctx.token_req = view("tokens"), view("positions"), view("token_req")
-        ctx.state_slots = view("state_slots")
+        ctx.state_slots, ctx.req_rows = view("state_slots"), view("req_rows")
+        ctx.embedding_state = engine.storage.state.get("embedding")
         ctx.want_rows, ctx.n_want, ctx.want_rows_identity = view("want_rows"), R, True
         ctx.decode_rows, ctx.n_decode_rows, ctx.decode_rows_identity = None, R, True
         ctx.prefill_tiles, ctx.n_prefill_tiles = None, 0

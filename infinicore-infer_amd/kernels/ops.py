@@ -835,3 +835,227 @@ def attention_span_prefill(q, out, gate, kcache, vcache, block_tables, tiles, n_
         block_tables.data_ptr(), block_tables.stride(0), tiles.data_ptr(), n_tiles, n_heads, n_kv_heads, key_dim, value_dim,
         page_size, float(scale), int(window or 0), int(keep_first or 0), int(bool(sink)), _stream()),
         "attention_span_prefill")
+
+
+# ---- several residual streams, the embedding with a pair table -----------------------------------------------
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+def pair_rows(tokens, positions, token_req, state_slots, prev_state, rows, buckets: int, mul_prev: int, mul_cur: int):
+    """rows[t] = (prev * mul_prev + tokens[t] * mul_cur) mod buckets, prev the token before in the same sequence (the
+    request's remembered token for a step's first row); ``buckets`` itself at position 0."""
+    _dev(tokens, positions, token_req, state_slots, prev_state, rows)
+    for t, n in ((tokens, "tokens"), (positions, "positions"), (token_req, "token_req"), (state_slots, "state_slots"),
+                 (prev_state, "prev_state"), (rows, "rows")):
+        _i32(t, n)
+    T = tokens.numel()
+    _need(positions.numel() == T and token_req.numel() == T and rows.numel() >= T, "pair_rows: T mismatch")
+    check(get_lib().ic_pair_rows(tokens.data_ptr(), positions.data_ptr(), token_req.data_ptr(), state_slots.data_ptr(),
+                                 prev_state.data_ptr(), rows.data_ptr(), T, int(buckets), int(mul_prev), int(mul_cur),
+                                 _stream()), "pair_rows")
+    return rows
+
+
+def embed_streams(tokens, table, out, rows=None, pair_table=None, token_req=None, state_slots=None, prev_state=None):
+    """out[s, t] = table[tokens[t]] + pair_table[rows[t]] for every stream s of out [S, T, d] (float32); with
+    ``prev_state`` the last token of every request's share of the step is remembered there."""
+    _dev(tokens, table, out, rows, pair_table, token_req, state_slots, prev_state)
+    _i32(tokens, "tokens")
+    _need(out.dim() == 3 and out.dtype == torch.float32 and out.is_contiguous(), "embed_streams: out is float32 [S, T, d]")
+    S, T, d = out.shape
+    _need(tokens.numel() == T and table.dim() == 2 and table.shape[1] == d and table.is_contiguous(), "embed_streams: table")
+    if pair_table is not None:
+        _i32(rows, "rows")
+        _need(pair_table.dtype == table.dtype and pair_table.shape[1] == d and pair_table.is_contiguous()
+              and rows.numel() >= T, "embed_streams: pair table")
+    if prev_state is not None:
+        for t, n in ((token_req, "token_req"), (state_slots, "state_slots"), (prev_state, "prev_state")):
+            _i32(t, n)
+    check(get_lib().ic_embed_streams(tokens.data_ptr(), _ptr(rows) if pair_table is not None else None, table.data_ptr(),
+                                     _ptr(pair_table), dtype_code(table.dtype), out.data_ptr(), S, T, d, _ptr(token_req),
+                                     _ptr(state_slots), _ptr(prev_state), _stream()), "embed_streams")
+    return out
+
+
+def hc_step(x, y=None, mix=None, out_w=None, in_w=None, norm_w=None, eps: float = 0.0, h=None):
+    """x [S, T, d] float32 streams.  With ``y`` [T, d]: x_t <- sum_s mix[s, t] x_s + out_w[t] y, all streams at once.
+    With ``in_w``: h = sum_s in_w[s] x_s (after the write), times rsqrt(mean + eps) * norm_w when ``norm_w`` is given."""
+    _dev(x, y, mix, out_w, in_w, norm_w, h)
+    _need(x.dim() == 3 and x.dtype == torch.float32 and x.is_contiguous(), "hc_step: x is float32 [S, T, d]")
+    S, T, d = x.shape
+    for v, n, shape in ((mix, "mix", (S, S)), (out_w, "out_w", (S,)), (in_w, "in_w", (S,)), (norm_w, "norm_w", (d,))):
+        if v is not None:
+            _need(v.dtype == torch.float32 and v.is_contiguous() and tuple(v.shape) == shape, "hc_step: %s is float32 %s" % (n, shape))
+    if y is not None:
+        _need(tuple(y.shape) == (T, d) and y.is_contiguous() and mix is not None and out_w is not None, "hc_step: y")
+    if in_w is not None:
+        _need(h is not None and tuple(h.shape) == (T, d) and h.is_contiguous(), "hc_step: h")
+    check(get_lib().ic_hc_step(x.data_ptr(), S, T, d, _ptr(y), dtype_code(y.dtype) if y is not None else 0, _ptr(mix),
+                               _ptr(out_w), _ptr(in_w), _ptr(norm_w), float(eps), _ptr(h),
+                               dtype_code(h.dtype) if h is not None else 0, _stream()), "hc_step")
+    return h
+
+
+# ---- mixers with a fixed-size state ------------------------------------------------------------------------------
+def _state_part(state, offset: int):
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous(), "state is float32 [slots, n]")
+    return state.data_ptr() + 4 * int(offset), state.shape[1]
+
+
+def causal_conv(xin, w, b, out, state, state_offset: int, token_req, req_start, state_slots, n_requests: int,
+                in_bias=None, out_copy=None, act: str = "none"):
+    """out[t, c] = act(b[c] + sum_k w[c, k] in(t - (taps-1-k), c)), in = xin + in_bias, rows before a request's first
+    one from its state (the last taps-1 inputs at ``state_offset``, [taps-1, C]), which is then moved on."""
+    _dev(xin, w, b, out, state, token_req, req_start, state_slots, in_bias, out_copy)
+    T, C = out.shape
+    taps = w.shape[1]
+    _need(xin.shape[0] == T and xin.shape[1] == C and xin.stride(1) == 1, "causal_conv: xin")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and w.dtype == torch.float32 and w.is_contiguous()
+          and tuple(w.shape) == (C, taps), "causal_conv: layout")
+    for v in (b, in_bias):
+        if v is not None:
+            _need(v.dtype == torch.float32 and v.numel() == C and v.is_contiguous(), "causal_conv: bias")
+    if out_copy is not None:
+        _need(out_copy.dtype == xin.dtype and tuple(out_copy.shape) == (T, C) and out_copy.stride(1) == 1, "causal_conv: copy")
+    for t, n in ((token_req, "token_req"), (req_start, "req_start"), (state_slots, "state_slots")):
+        _i32(t, n)
+    _need(token_req.numel() >= T and req_start.numel() >= n_requests + 1 and state_slots.numel() >= n_requests, "causal_conv: lists")
+    sp, stride = _state_part(state, state_offset)
+    _need(state_offset + (taps - 1) * C <= stride, "causal_conv: state too small")
+    check(get_lib().ic_causal_conv(xin.data_ptr(), xin.stride(0), dtype_code(xin.dtype), _ptr(in_bias), w.data_ptr(), _ptr(b),
+                                   taps, C, out.data_ptr(), _ptr(out_copy), out_copy.stride(0) if out_copy is not None else 0,
+                                   {"none": 0, "silu": 1}[act], sp, stride, token_req.data_ptr(), req_start.data_ptr(),
+                                   state_slots.data_ptr(), T, n_requests, _stream()), "causal_conv")
+    return out
+
+
+def rglru_scan(gates, gate_bias, u, yb, y_bias, decay, block_width: int, out, state, state_offset: int, req_start,
+               state_slots, n_requests: int):
+    """The gated diagonal recurrence over every request's rows (see csrc/recurrent.hip); out = S * gelu_tanh(yb + y_bias)."""
+    _dev(gates, gate_bias, u, yb, y_bias, decay, out, state, req_start, state_slots)
+    T, width = u.shape
+    for v, shape in ((gates, (T, 2 * width)), (u, (T, width))):
+        _need(v.dtype == torch.float32 and v.is_contiguous() and tuple(v.shape) == shape, "rglru_scan: float32 operands")
+    for v, n in ((gate_bias, 2 * width), (decay, width), (y_bias, width)):
+        _need(v is None or (v.dtype == torch.float32 and v.numel() == n and v.is_contiguous()), "rglru_scan: vectors")
+    _need(tuple(yb.shape) == (T, width) and yb.stride(1) == 1 and out.dtype == yb.dtype and tuple(out.shape) == (T, width)
+          and out.is_contiguous(), "rglru_scan: branches")
+    _i32(req_start, "req_start")
+    _i32(state_slots, "state_slots")
+    sp, stride = _state_part(state, state_offset)
+    _need(state_offset + width <= stride, "rglru_scan: state too small")
+    check(get_lib().ic_rglru_scan(gates.data_ptr(), gate_bias.data_ptr(), u.data_ptr(), yb.data_ptr(), yb.stride(0),
+                                  dtype_code(yb.dtype), _ptr(y_bias), decay.data_ptr(), width, int(block_width), out.data_ptr(),
+                                  sp, stride, req_start.data_ptr(), state_slots.data_ptr(), n_requests, _stream()), "rglru_scan")
+    return out
+
+
+def ssm_scan(xbc, dt_raw, dt_bias, neg_a, d_skip, heads: int, head_dim: int, state_dim: int, groups: int, y, state,
+             state_offset: int, req_start, state_slots, n_requests: int):
+    """The state-space recurrence over every request's rows (see csrc/recurrent.hip): y float32 [T, heads * head_dim]."""
+    _dev(xbc, dt_raw, dt_bias, neg_a, d_skip, y, state, req_start, state_slots)
+    T = xbc.shape[0]
+    inner = heads * head_dim
+    _need(xbc.dtype == torch.float32 and xbc.is_contiguous() and xbc.shape[1] == inner + 2 * groups * state_dim, "ssm_scan: xbc")
+    _need(y.dtype == torch.float32 and y.is_contiguous() and tuple(y.shape) == (T, inner), "ssm_scan: y")
+    _need(tuple(dt_raw.shape) == (T, heads) and dt_raw.stride(1) == 1, "ssm_scan: dt")
+    for v in (dt_bias, neg_a, d_skip):
+        _need(v.dtype == torch.float32 and v.numel() == heads and v.is_contiguous(), "ssm_scan: per-head vectors")
+    _i32(req_start, "req_start")
+    _i32(state_slots, "state_slots")
+    sp, stride = _state_part(state, state_offset)
+    _need(state_offset + inner * state_dim <= stride, "ssm_scan: state too small")
+    check(get_lib().ic_ssm_scan(xbc.data_ptr(), dt_raw.data_ptr(), dt_raw.stride(0), dtype_code(dt_raw.dtype), dt_bias.data_ptr(),
+                                neg_a.data_ptr(), d_skip.data_ptr(), heads, head_dim, state_dim, groups, y.data_ptr(), sp, stride,
+                                req_start.data_ptr(), state_slots.data_ptr(), n_requests, _stream()), "ssm_scan")
+    return y
+
+
+def gated_group_norm(y, z, weight, groups: int, eps: float, out):
+    """out = rms_in_groups(y * silu(z)) * weight; y float32 [T, n], z and out the compute dtype."""
+    _dev(y, z, weight, out)
+    T, n = y.shape
+    _need(y.dtype == torch.float32 and y.is_contiguous() and tuple(z.shape) == (T, n) and z.stride(1) == 1
+          and out.dtype == z.dtype and tuple(out.shape) == (T, n) and out.is_contiguous(), "gated_group_norm: layout")
+    _need(weight.dtype == torch.float32 and weight.numel() == n and weight.is_contiguous(), "gated_group_norm: weight")
+    check(get_lib().ic_gated_group_norm(y.data_ptr(), z.data_ptr(), z.stride(0), dtype_code(z.dtype), weight.data_ptr(), n,
+                                        int(groups), float(eps), out.data_ptr(), T, _stream()), "gated_group_norm")
+    return out
+
+
+def blocked_product(a, w, out, gate=None):
+    """out[m, b, n] = sum_k a[m, b, k] w[b, n, k] (times sigmoid(gate[m, b, n])): a [M, B, K] and out [M, B, N] may be
+    views whose rows are strided; w [B, N, K] contiguous.  out may be float32 under bfloat16 operands."""
+    _dev(a, w, out, gate)
+    M, B, K = a.shape
+    N = w.shape[1]
+    _need(tuple(w.shape) == (B, N, K) and w.is_contiguous() and w.dtype == a.dtype, "blocked_product: w")
+    _need(tuple(out.shape) == (M, B, N) and a.stride(2) == 1 and out.stride(2) == 1, "blocked_product: shapes")
+    if gate is not None:
+        _need(tuple(gate.shape) == (M, B, N) and gate.dtype == a.dtype and gate.stride(2) == 1 and gate.stride(1) == out.stride(1),
+              "blocked_product: gate")
+    check(get_lib().ic_blocked_product(a.data_ptr(), a.stride(0), a.stride(1), w.data_ptr(), dtype_code(a.dtype), out.data_ptr(),
+                                       dtype_code(out.dtype), out.stride(0), out.stride(1), _ptr(gate),
+                                       gate.stride(0) if gate is not None else 0, M, N, K, B, _stream()), "blocked_product")
+    return out
+
+
+# ---- attention through a latent -------------------------------------------------------------------------------------
+def latent_prep(rows, q_rank: int, kv_rank: int, rot_dim: int, qn_w, kvn_w, eps: float, freq, rot_dims: int, positions,
+                cq, cache, slots):
+    """cq = rms(rows[:, :q_rank]) * qn_w; cache[slots[t]] = [rms(next kv_rank columns) * kvn_w | the next rot_dim rotated]."""
+    _dev(rows, qn_w, kvn_w, freq, positions, cq, cache, slots)
+    T = rows.shape[0]
+    _need(rows.stride(1) == 1 and rows.shape[1] >= q_rank + kv_rank + rot_dim, "latent_prep: rows")
+    _need(cq.dtype == rows.dtype and tuple(cq.shape) == (T, q_rank) and cq.is_contiguous(), "latent_prep: cq")
+    for v, n in ((qn_w, q_rank), (kvn_w, kv_rank), (freq, rot_dims // 2)):
+        _need(v.dtype == torch.float32 and v.numel() >= n and v.is_contiguous(), "latent_prep: vectors")
+    _i32(positions, "positions")
+    if slots is not None:
+        _i32(slots, "slots")
+        _need(cache.dtype == rows.dtype and cache.is_contiguous() and cache.shape[-1] == kv_rank + rot_dim and cache.shape[1] == 1,
+              "latent_prep: cache plane")
+    check(get_lib().ic_latent_prep(rows.data_ptr(), rows.stride(0), dtype_code(rows.dtype), q_rank, kv_rank, rot_dim,
+                                   qn_w.data_ptr(), kvn_w.data_ptr(), float(eps), freq.data_ptr(), int(rot_dims),
+                                   positions.data_ptr(), cq.data_ptr(), _ptr(cache), _ptr(slots), T, _stream()), "latent_prep")
+
+
+def latent_q_rotate(q, dim: int, rot_dim: int, kv_rank: int, heads: int, freq, rot_dims: int, positions, qa):
+    """qa[t, h, kv_rank:] = the rotated part q[t, h, dim:] turned by its position's angles."""
+    _dev(q, freq, positions, qa)
+    T = q.shape[0]
+    _need(q.shape[1] == heads * (dim + rot_dim) and q.stride(1) == 1 and qa.dtype == q.dtype
+          and tuple(qa.shape) == (T, heads * (kv_rank + rot_dim)) and qa.stride(1) == 1, "latent_q_rotate: layout")
+    _i32(positions, "positions")
+    check(get_lib().ic_latent_q_rotate(q.data_ptr(), q.stride(0), dtype_code(q.dtype), dim, rot_dim, kv_rank, heads,
+                                       freq.data_ptr(), int(rot_dims), positions.data_ptr(), qa.data_ptr(), qa.stride(0), T,
+                                       _stream()), "latent_q_rotate")
+
+
+LATENT_MAX_RANK = 512
+
+
+def attention_latent(qa, out, cache, block_tables, token_req, positions, heads: int, kv_rank: int, rot_dim: int,
+                     page_size: int, scale: float, n_split: int = 1, part_acc=None, part_ml=None):
+    """out[t, h, :kv_rank] = sum_j p_j c_j over the cached rows [c | k_rot] j <= positions[t] of the token's request,
+    p = softmax(scale * qa[t, h] . row_j): every head walks the same rows."""
+    _dev(qa, out, cache, block_tables, token_req, positions, part_acc, part_ml)
+    T = qa.shape[0]
+    D = kv_rank + rot_dim
+    _need(tuple(qa.shape) == (T, heads * D) and qa.stride(1) == 1 and out.dtype == qa.dtype
+          and tuple(out.shape) == (T, heads * kv_rank) and out.stride(1) == 1, "attention_latent: q / out")
+    _need(cache.dtype == qa.dtype and cache.is_contiguous() and cache.shape[-1] == D and cache.shape[1] == 1
+          and cache.shape[2] == page_size, "attention_latent: cache plane")
+    for t, n in ((block_tables, "block_tables"), (token_req, "token_req"), (positions, "positions")):
+        _need(t.dtype == torch.int32, n + " must be int32")
+    _need(block_tables.stride(1) == 1 and token_req.numel() >= T and positions.numel() >= T, "attention_latent: lists")
+    if n_split > 1:
+        _need(part_acc is not None and part_ml is not None and part_acc.dtype == torch.float32 and part_ml.dtype == torch.float32
+              and part_acc.numel() >= T * heads * n_split * kv_rank and part_ml.numel() >= T * heads * n_split * 2,
+              "attention_latent: scratch too small")
+    check(get_lib().ic_attn_latent(qa.data_ptr(), qa.stride(0), out.data_ptr(), out.stride(0), dtype_code(qa.dtype),
+                                   cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(),
+                                   positions.data_ptr(), T, heads, kv_rank, rot_dim, page_size, float(scale), int(n_split),
+                                   _ptr(part_acc), _ptr(part_ml), _stream()), "attention_latent")
+    return out

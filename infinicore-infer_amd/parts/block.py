@@ -10,6 +10,10 @@ it: the block leaves its last add pending for whoever normalises next.  For
 few rows the add and the norm go further, into the products on either side
 (``ResidualTail`` / ``DeferredRows``): then a layer is six kernels, not eight.
 """
+import torch
+
+from ..kernels import ops
+from ..weights.loader import WeightSpec
 from .base import Block, DeferredRows, ResidualTail, StreamCopy, register_part
 
 
@@ -124,3 +128,85 @@ class OutputNormResidualBlock(Block):
             y = self.feed_forward.forward(h, ctx)
             self.feed_forward_norm.forward_into_stream(y, x, copy=copy)
         return StreamCopy(h)
+
+
+class OwedStreamWrite:
+    """The write of a sublayer's result into several residual streams, still owed: the next read of the streams (the
+    next sublayer's input, in whichever block) does it in the same kernel.  Whoever cannot, settles it."""
+
+    def __init__(self, y, mix, out_w):
+        self.y, self.mix, self.out_w = y, mix, out_w
+
+    def settle(self, x, ctx=None):
+        ops.hc_step(x, y=self.y, mix=self.mix, out_w=self.out_w)
+        return None
+
+
+@register_part("block", "hyper_connections")
+class HyperConnectionBlock(Block):
+    """Pre-norm sublayers over ``streams`` float32 copies of the residual stream x_1..x_S ([S, T, d]).  Sublayer q
+    (1: the mixer, 2: the feed-forward) reads u = sum_s in_q[s] x_s, computes y = f(norm_q(u)), and rewrites all streams
+    at once from the old ones: x_t <- sum_s mix_q[s, t] x_s + out_q[t] y.  Tensors: ``hc<q>.in`` [S], ``hc<q>.out`` [S],
+    ``hc<q>.mix`` [S, S] ([from, to]), held in float32.  One row kernel per sublayer does the write owed by the
+    sublayer before, the read, and the norm."""
+    graph_safe = True
+    accepts_owed_update = True
+
+    def __init__(self, name, runtime, mixer=None, mixer_norm=None, feed_forward=None, feed_forward_norm=None, streams: int = 2):
+        super().__init__(name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm)
+        if mixer is None or mixer_norm is None:
+            raise ValueError("block %s: a hyper-connection block needs a mixer and its norm" % name)
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("block %s: a feed-forward and its norm come together, or neither" % name)
+        for n in (mixer_norm, feed_forward_norm):
+            if n is not None and n.deferred() is None:
+                raise ValueError("block %s: norm part %s is not a weighted RMS norm" % (name, type(n).__name__))
+        self.streams = int(streams)
+        if not 1 <= self.streams <= 8:
+            raise ValueError("block %s: 1..8 residual streams (got %d)" % (name, self.streams))
+        self.hc = {}
+
+    def _subs(self):
+        return (1, 2) if self.feed_forward is not None else (1,)
+
+    def weight_specs(self):
+        S, specs = self.streams, {}
+        for q in self._subs():
+            p = "%shc%d." % (self.name, q)
+            specs[p + "in"] = WeightSpec((S,), "vector")
+            specs[p + "out"] = WeightSpec((S,), "vector")
+            specs[p + "mix"] = WeightSpec((S, S), "vector")
+        return specs
+
+    def load_weights(self, tensors):
+        for q in self._subs():
+            p = "%shc%d." % (self.name, q)
+            self.hc[q] = tuple(tensors[p + k].to(torch.float32).contiguous() for k in ("in", "out", "mix"))
+
+    def _read(self, x, pending, q, norm, ctx):
+        """The sublayer's input: the owed write (if any), the read and the norm in one kernel."""
+        T, d = x.shape[1], x.shape[2]
+        h = ctx.ws.buffer("normed", (T, d), self.runtime.dtype)
+        w, eps = norm.deferred()
+        if isinstance(pending, OwedStreamWrite):
+            ops.hc_step(x, y=pending.y, mix=pending.mix, out_w=pending.out_w, in_w=self.hc[q][0], norm_w=w, eps=eps, h=h)
+        else:
+            ops.hc_step(x, in_w=self.hc[q][0], norm_w=w, eps=eps, h=h)
+        return h
+
+    def forward(self, x, pending, ctx, cache):
+        if x.dim() != 3 or x.shape[0] != self.streams:
+            raise RuntimeError("block %s wants the residual stream as [%d, T, d]" % (self.name, self.streams))
+        if pending is not None and not isinstance(pending, OwedStreamWrite):
+            if isinstance(pending, StreamCopy):
+                pending = None
+            else:
+                raise RuntimeError("block %s was handed a pending add of another kind of block" % self.name)
+        h = self._read(x, pending, 1, self.mixer_norm, ctx)
+        y = self.mixer.forward(h, ctx, cache)
+        pending = OwedStreamWrite(y, self.hc[1][2], self.hc[1][1])
+        if self.feed_forward is not None:
+            h = self._read(x, pending, 2, self.feed_forward_norm, ctx)
+            y = self.feed_forward.forward(h, ctx)
+            pending = OwedStreamWrite(y, self.hc[2][2], self.hc[2][1])
+        return pending

@@ -52,6 +52,11 @@ class DecoderModel:
             if not e.writes_cache and e.cache not in writers:
                 raise ValueError("cache slot %d is read but never written" % e.cache)
         self._writers = writers
+        self.streams = int(getattr(spec, "residual_streams", 1) or 1)
+        if self.streams > 1:
+            for l in self.layers:
+                if getattr(l, "streams", 1) != self.streams:
+                    raise ValueError("block %s keeps %d residual streams, the model %d" % (l.name, getattr(l, "streams", 1), self.streams))
         # an entry that reads another entry's cache must fit what the writer keeps: the same heads and
         # head size, and no more keys than the writer's window holds (pages behind a window are given
         # back and their block-table entries are reused)
@@ -118,6 +123,11 @@ class DecoderModel:
             needs[slot] = self._cache_need_of(layer)
         return needs
 
+    def embedding_cache_need(self) -> CacheNeed:
+        """What the embedding keeps per request (the token before a step's first one, for a table of pairs), or nothing."""
+        need = getattr(self.embedding, "cache_need", None)
+        return need() if need is not None else CacheNeed()
+
     def weight_bytes(self) -> int:
         seen, total = set(), 0
         for p in self.all_parts():
@@ -131,7 +141,8 @@ class DecoderModel:
     def forward(self, ctx):
         """Runs ctx.T tokens; returns float32 logits [len(ctx.want_rows), vocab] or None."""
         T = ctx.T
-        x = ctx.ws.buffer("residual", (T, self.spec.hidden_size), torch.float32)
+        shape = (T, self.spec.hidden_size) if self.streams == 1 else (self.streams, T, self.spec.hidden_size)
+        x = ctx.ws.buffer("residual", shape, torch.float32)
         if getattr(self.embedding, "takes_context", False):
             pending = self.embedding.forward(ctx.tokens, x, ctx)      # may hand on the stream's copy (StreamCopy)
         else:
@@ -140,12 +151,16 @@ class DecoderModel:
         last = len(self.schedule) - 1
         for i, e in enumerate(self.schedule):
             block = self.layers[e.layer]
+            if hasattr(pending, "settle") and not getattr(block, "accepts_owed_update", False):
+                pending = pending.settle(x, ctx)                      # an update only its own kind of block can fuse
             if isinstance(pending, StreamCopy) and not getattr(block, "accepts_stream_copy", False):
                 pending = None                                        # nothing is owed; this block makes its own input
             if not block.fuses_successor:
                 if isinstance(pending, DeferredRows):
                     raise RuntimeError("block %s was handed half-normed rows it did not ask for" % block.name)
                 pending = block.forward(x, pending, ctx, ctx.cache_view(e))
+                if ctx.layer_probe is not None:
+                    ctx.layer_probe(i, x, pending)
                 continue
             # the norm that runs next, if whoever applies it can take its rows half done
             if i < last:
@@ -155,8 +170,17 @@ class DecoderModel:
             else:
                 successor = None
             pending = block.forward(x, pending, ctx, ctx.cache_view(e), successor=successor)
+            if ctx.layer_probe is not None:
+                ctx.layer_probe(i, x, pending)
+        if hasattr(pending, "settle"):
+            pending = pending.settle(x, ctx)
+        if ctx.layer_probe is not None:
+            ctx.layer_probe(len(self.schedule), x, pending)
         if ctx.n_want == 0:
             return None
+        if self.streams > 1:
+            # the streams' sum is what the final norm reads
+            x = ops.hc_step(x, in_w=self._stream_ones(x), h=ctx.ws.buffer("residual_sum", (T, self.spec.hidden_size), torch.float32))
         if isinstance(pending, DeferredRows):
             return self.head.forward(pending, ctx.want_rows, self.final_norm, ctx)
         if isinstance(pending, StreamCopy):
@@ -164,6 +188,13 @@ class DecoderModel:
         if pending is not None:
             ops.residual_add(x, pending[0], pending[1])
         return self.head.forward(x, ctx.want_rows, self.final_norm, ctx)
+
+
+    def _stream_ones(self, x):
+        ones = getattr(self, "_ones", None)
+        if ones is None or ones.device != x.device:
+            ones = self._ones = torch.ones(self.streams, dtype=torch.float32, device=x.device)
+        return ones
 
 
 def build_model(spec: ModelSpec, runtime: Runtime) -> DecoderModel:

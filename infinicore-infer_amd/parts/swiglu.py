@@ -19,19 +19,22 @@ class SwiGLU(FeedForward):
     accepts_deferred = True
     fuses_tail = True
 
-    def __init__(self, name, runtime, hidden_size: int, intermediate_size: int):
+    def __init__(self, name, runtime, hidden_size: int, intermediate_size: int, gate_name: str = "gate_proj.weight",
+                 up_name: str = "up_proj.weight", down_name: str = "down_proj.weight"):
+        """``gate_name`` / ``up_name`` / ``down_name``: the matrices' names after the part's prefix."""
         super().__init__(name, runtime)
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
+        self.gate_name, self.up_name, self.down_name = name + gate_name, name + up_name, name + down_name
         self.w_gate_up = None
         self.w_down = None
 
     def weight_specs(self):
         n, d, di = self.name, self.hidden_size, self.intermediate_size
         return {
-            n + "gate_proj.weight": WeightSpec((di, d), pack=(n + "gate_up_proj.packed", 0)),
-            n + "up_proj.weight": WeightSpec((di, d), pack=(n + "gate_up_proj.packed", 1)),
-            n + "down_proj.weight": WeightSpec((d, di)),
+            self.gate_name: WeightSpec((di, d), pack=(n + "gate_up_proj.packed", 0)),
+            self.up_name: WeightSpec((di, d), pack=(n + "gate_up_proj.packed", 1)),
+            self.down_name: WeightSpec((d, di)),
         }
 
     def load_weights(self, tensors):
@@ -40,11 +43,11 @@ class SwiGLU(FeedForward):
         if packed is not None:
             self.w_gate_up = packed
         else:
-            g, u = tensors[n + "gate_proj.weight"], tensors[n + "up_proj.weight"]
+            g, u = tensors[self.gate_name], tensors[self.up_name]
             if g.dtype != u.dtype:
                 g, u = g.to(torch.float32), u.to(torch.float32)
             self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
-        self.w_down = tensors[n + "down_proj.weight"]
+        self.w_down = tensors[self.down_name]
 
     def native_desc(self):
         from ..kernels.lib import IcSwiGLU
