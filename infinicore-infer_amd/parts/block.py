@@ -138,7 +138,7 @@ class OwedStreamWrite:
         self.y, self.mix, self.out_w = y, mix, out_w
 
     def settle(self, x, ctx=None):
-        ops.hc_step(x, y=self.y, mix=self.mix, out_w=self.out_w)
+        ops.hc_step(x if x.dim() == 3 else x.unsqueeze(0), y=self.y, mix=self.mix, out_w=self.out_w)
         return None
 
 
@@ -173,9 +173,10 @@ class HyperConnectionBlock(Block):
         S, specs = self.streams, {}
         for q in self._subs():
             p = "%shc%d." % (self.name, q)
-            specs[p + "in"] = WeightSpec((S,), "vector")
+            # (random-weights mode draws them around means that keep the streams' size: the read and the mix average)
+            specs[p + "in"] = WeightSpec((S,), "vector", mean=1.0 / S)
             specs[p + "out"] = WeightSpec((S,), "vector")
-            specs[p + "mix"] = WeightSpec((S, S), "vector")
+            specs[p + "mix"] = WeightSpec((S, S), "vector", mean=1.0 / S)
         return specs
 
     def load_weights(self, tensors):
@@ -195,6 +196,8 @@ class HyperConnectionBlock(Block):
         return h
 
     def forward(self, x, pending, ctx, cache):
+        if x.dim() == 2 and self.streams == 1:
+            x = x.unsqueeze(0)                        # one stream: the model keeps it as [T, d]
         if x.dim() != 3 or x.shape[0] != self.streams:
             raise RuntimeError("block %s wants the residual stream as [%d, T, d]" % (self.name, self.streams))
         if pending is not None and not isinstance(pending, OwedStreamWrite):

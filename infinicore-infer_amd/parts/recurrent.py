@@ -43,7 +43,7 @@ class GatedLinearRecurrence(Mixer):
         return {
             n + "y": WeightSpec((w, d), pack=(pack, 0)), n + "x": WeightSpec((w, d), pack=(pack, 1)),
             n + "y.b": WeightSpec((w,), "vector", mean=0.0), n + "x.b": WeightSpec((w,), "vector", mean=0.0),
-            n + "conv": WeightSpec((w, self.taps), "vector", mean=0.0), n + "conv.b": WeightSpec((w,), "vector", mean=0.0),
+            n + "conv": WeightSpec((w, self.taps), "vector", mean=1.0 / self.taps), n + "conv.b": WeightSpec((w,), "vector", mean=0.0),
             n + "ra": WeightSpec((b, bw, bw)), n + "ri": WeightSpec((b, bw, bw)),
             n + "ra.b": WeightSpec((b, bw), "vector", mean=0.0), n + "ri.b": WeightSpec((b, bw), "vector", mean=0.0),
             n + "lam": WeightSpec((w,), "vector", mean=0.0),
@@ -116,7 +116,7 @@ class StateSpaceMixer(Mixer):
         n, d = self.name, self.hidden_size
         return {
             n + "in": WeightSpec((self.proj, d)),
-            n + "conv": WeightSpec((self.channels, self.taps), "vector", mean=0.0),
+            n + "conv": WeightSpec((self.channels, self.taps), "vector", mean=1.0 / self.taps),
             n + "conv.b": WeightSpec((self.channels,), "vector", mean=0.0),
             n + "dt_bias": WeightSpec((self.heads,), "vector", mean=0.0),
             n + "A_log": WeightSpec((self.heads,), "vector", mean=0.0),

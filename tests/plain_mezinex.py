@@ -209,3 +209,75 @@ def forward(cfg, W, tokens, dtype=torch.float64, layer_outputs=None):
     if streams:
         x = xs.sum(0)
     return (rms(x, eps) * W["final.norm"]) @ W["head"].T * cfg.get("logit_scale", 1.0)
+
+
+# ---- weights for the tests ----------------------------------------------------------------------------------------
+def tensor_shapes(cfg):
+    """Name -> shape of every tensor of a configuration."""
+    d, V = cfg["width"], cfg["vocab"]
+    S = cfg.get("streams")
+    out = {"embed": (V, d), "final.norm": (d,), "head": (V, d)}
+    big = (cfg.get("embedding") or {}).get("bigram")
+    if big:
+        out["bigram"] = (big["buckets"] + 1, d)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = "l%d." % i, l["mixer"]
+        out[p + "norm1"] = (d,)
+        if l["type"] == "rglru":
+            w, b = m["width"], m["blocks"]
+            out.update({p + "mix.y": (w, d), p + "mix.y.b": (w,), p + "mix.x": (w, d), p + "mix.x.b": (w,),
+                        p + "mix.conv": (w, m["conv"]), p + "mix.conv.b": (w,), p + "mix.ra": (b, w // b, w // b),
+                        p + "mix.ra.b": (b, w // b), p + "mix.ri": (b, w // b, w // b), p + "mix.ri.b": (b, w // b),
+                        p + "mix.lam": (w,), p + "mix.o": (d, w)})
+        elif l["type"] == "mamba2":
+            inner, gn = m["heads"] * m["vdim"], m["groups"] * m["state"]
+            out.update({p + "mix.in": (2 * inner + 2 * gn + m["heads"], d), p + "mix.conv": (inner + 2 * gn, m["conv"]),
+                        p + "mix.conv.b": (inner + 2 * gn,), p + "mix.dt_bias": (m["heads"],), p + "mix.A_log": (m["heads"],),
+                        p + "mix.D": (m["heads"],), p + "mix.norm": (inner,), p + "mix.o": (d, inner)})
+        else:
+            H = m["heads"]
+            out.update({p + "mix.dq": (m["q_rank"], d), p + "mix.dq.norm": (m["q_rank"],),
+                        p + "mix.uq": (H * (m["dim"] + m["rot_dim"]), m["q_rank"]),
+                        p + "mix.dkv": (m["kv_rank"] + m["rot_dim"], d), p + "mix.dkv.norm": (m["kv_rank"],),
+                        p + "mix.uk": (H * m["dim"], m["kv_rank"]), p + "mix.uv": (H * m["vdim"], m["kv_rank"]),
+                        p + "mix.g": (H * m["vdim"], d), p + "mix.o": (d, H * m["vdim"])})
+        subs = [1]
+        if l.get("mlp"):
+            ff = l["mlp"]["ff"]
+            out.update({p + "norm2": (d,), p + "mlp.gate": (ff, d), p + "mlp.up": (ff, d), p + "mlp.down": (d, ff)})
+            subs.append(2)
+        if S:
+            for q in subs:
+                out.update({p + "hc%d.in" % q: (S,), p + "hc%d.out" % q: (S,), p + "hc%d.mix" % q: (S, S)})
+    return out
+
+
+def random_weights(cfg, seed):
+    """Weights at scales that keep every mechanism alive: products near unit gain, decays spread over (0, 1), streams
+    that mix but do not blow up.  Values are rounded to bfloat16 (what a folder stores)."""
+    g = torch.Generator().manual_seed(seed)
+    S = cfg.get("streams") or 1
+    W = {}
+    for name, shape in tensor_shapes(cfg).items():
+        r = torch.randn(*shape, generator=g, dtype=torch.float64)
+        leaf = name.split(".", 1)[1] if name.startswith("l") and "." in name else name
+        if leaf in ("norm1", "norm2", "mix.norm", "mix.dq.norm", "mix.dkv.norm", "mix.D") or name == "final.norm":
+            t = 1.0 + 0.2 * r
+        elif leaf.endswith(".b") or leaf in ("mix.dt_bias", "mix.A_log"):
+            t = 0.5 * r
+        elif leaf == "mix.lam":
+            t = 1.5 * r - 1.0
+        elif leaf == "mix.conv":
+            t = 0.6 * r
+        elif leaf.endswith(".in"):
+            t = 1.0 / S + 0.3 * r
+        elif leaf.endswith(".out"):
+            t = 1.0 + 0.3 * r
+        elif leaf.endswith(".mix"):
+            t = torch.eye(S, dtype=torch.float64) + 0.15 * r
+        elif name in ("embed", "bigram"):
+            t = r
+        else:
+            t = r / math.sqrt(shape[-1])
+        W[name] = t.to(torch.bfloat16).to(torch.float64)
+    return W
