@@ -12,9 +12,9 @@ seeded uniform-random token ids.  One JSON line is printed.
   --workload mixed   the 1B shape's workload: 64 requests, prompts of 128..2,048 tokens, portions of 512
   --workload long    the 8B shape's workload: 4 prompts of 16,384 tokens, then decoding
   --direct           decode by calling the step function directly, without the scheduler
-  --workload designs the Fopezen decoder beside the MiniCPM decoder at equal layer sizes (a few layers of three real
+  --workload designs the Fopezen and Mezinex decoders beside the MiniCPM decoder at equal layer sizes (a few layers of three real
                      models' sizes): prefill and decode throughput of both, with the fraction of the memory or
-                     matrix-core peak each reaches (--only fopezen|minicpm: one of them, for a profiler)
+                     matrix-core peak each reaches (--only fopezen|minicpm|mezinex: one of them, for a profiler)
 """
 import argparse
 import json
@@ -198,13 +198,30 @@ def _design_configs(z, layers):
     fop = dict(architecture="Fopezen", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-5),
                layers=[dict(type=kinds[i % 4], mixer=mixer(z["window"], z["keep"]), mlp=dict(kind="dense", ff=z["ff"]))
                        for i in range(layers)])
-    return {"minicpm": mini, "fopezen": fop}
+    # Mezinex at the same width and feed-forward: latent attention with the same heads and plain key size (a rotated part of
+    # 64 or 32, a latent of 512 or 256, a query latent of a third of the width), a gated linear recurrence as wide as the
+    # model with one gate block per head, a state-space mixer of twice the width in heads of 64 with states of 128; two
+    # residual streams and a pair table
+    big = z["dim"] >= 128
+    latent = dict(heads=z["heads"], dim=z["dim"], rot_dim=64 if big else 32, vdim=z["dim"], q_rank=z["width"] // 3 // 64 * 64,
+                  kv_rank=512 if big else 256, scale=(z["dim"] + (64 if big else 32)) ** -0.5,
+                  rot=dict(base=1000000.0, dims=64 if big else 32))
+    rglru = dict(width=z["width"], blocks=z["heads"], conv=4)
+    ssm = dict(heads=2 * z["width"] // 64, vdim=64, state=128, groups=8, norm_groups=8, conv=4)
+    mez_kinds = [("latent_attention", latent), ("rglru", rglru), ("mamba2", ssm), ("latent_attention", latent)]
+    mez = dict(architecture="Mezinex", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-5), logit_scale=1.0, streams=2,
+               embedding=dict(bigram=dict(buckets=65521, mul_prev=127, mul_cur=17)),
+               layers=[dict(type=mez_kinds[i % 4][0], mixer=mez_kinds[i % 4][1], mlp=dict(kind="dense", ff=z["ff"]))
+                       for i in range(layers)])
+    return {"minicpm": mini, "fopezen": fop, "mezinex": mez}
 
 
 def _design_numbers(design, z, layers, kinds=None):
     """(weight bytes a decode step reads, cache bytes a decode step reads per request at context n, prefill flops at T)."""
     d, H, G, dk, ff, V = z["width"], z["heads"], z["kv"], z["dim"], z["ff"], z["vocab"]
     eb = _elem_bytes()
+    if design == "mezinex":
+        return _mezinex_numbers(z, layers)
     if design == "minicpm":
         per_layer = (H + 2 * G) * dk * d + H * dk * d + 3 * d * ff
         kv = lambda n: 2 * layers * G * dk * eb * n
@@ -219,6 +236,39 @@ def _design_numbers(design, z, layers, kinds=None):
         attn = lambda T: layers * H * (dk + dv) * 2.0 * sum(seen(i + 1) for i in range(T))
     weights = eb * (layers * per_layer + V * d)
     return weights, kv, (lambda T: 2.0 * T * layers * per_layer + attn(T) + 2.0 * V * d)
+
+
+def _mezinex_numbers(z, layers):
+    """As ``_design_numbers`` for the Mezinex configuration of ``_design_configs``: weights a decode step reads, bytes of
+    cache and state it reads per request, flops of a prompt (products, the walk over the latent rows, the recurrences)."""
+    cfg = _design_configs(z, layers)["mezinex"]
+    d, ff, V, eb = z["width"], z["ff"], z["vocab"], _elem_bytes()
+    weights, per_tok_lin, cache_row, state_bytes = V * d, 0.0, 0.0, 0.0
+    walk = []          # (heads, row width + latent width) per attention layer: flops of the walk per (query, key) pair / 2
+    scan = 0.0         # flops per token of the recurrences
+    for l in cfg["layers"]:
+        m = l["mixer"]
+        n = 3 * d * ff
+        if l["type"] == "latent_attention":
+            H, R, E = m["heads"], m["kv_rank"], m["rot_dim"]
+            n += (m["q_rank"] + R + E + H * m["vdim"]) * d + H * (m["dim"] + E) * m["q_rank"] + H * m["dim"] * R + H * m["vdim"] * R + d * H * m["vdim"]
+            cache_row += (R + E) * eb
+            walk.append(H * (2 * R + E))
+        elif l["type"] == "rglru":
+            w = m["width"]
+            n += 3 * w * d + 2 * w * (w // m["blocks"])
+            state_bytes += 2 * 4 * w * m["conv"]
+            scan += 12.0 * w
+        else:
+            inner, gn = m["heads"] * m["vdim"], m["groups"] * m["state"]
+            n += (2 * inner + 2 * gn + m["heads"]) * d + d * inner
+            state_bytes += 2 * 4 * (inner * m["state"] + (m["conv"] - 1) * (inner + 2 * gn))
+            scan += 6.0 * inner * m["state"]
+        weights += n
+        per_tok_lin += 2.0 * n
+    kv = lambda n: cache_row * n + state_bytes
+    flops = lambda T: T * (per_tok_lin + scan) + sum(2.0 * w for w in walk) * (T * (T + 1) / 2) + 2.0 * V * d
+    return eb * weights, kv, flops
 
 
 def run_designs(args):
@@ -263,7 +313,7 @@ def run_designs(args):
             print(json.dumps(row), file=sys.stderr, flush=True)
             del engine, model
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "prefill and decode tokens/s of two decoder designs at equal layer sizes", "unit": "tokens/s",
+    print(json.dumps({"metric": "prefill and decode tokens/s of the decoder designs at equal layer sizes", "unit": "tokens/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": dname, "prompt": PROMPT,
                       "data": "synthetic (seeded random weights and token ids)", "rows": rows}))
     return 0
@@ -356,7 +406,7 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES), help="2b is the benchmark's configuration (default; 1b for --workload mixed)")
     ap.add_argument("--sizes", default=None, help="--workload designs: comma-separated sizes (default: all of 2b-like, 8b-like, 1b-like)")
-    ap.add_argument("--only", default=None, choices=["fopezen", "minicpm"], help="--workload designs: one design only")
+    ap.add_argument("--only", default=None, choices=["fopezen", "minicpm", "mezinex"], help="--workload designs: one design only")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long", "designs"],
                     help="decode: the benchmark (prefill of one prompt, decode steps at fixed batches); "
                          "mixed: 64 requests of 128..2048 prompt tokens through the scheduler, --steps tokens generated each; "

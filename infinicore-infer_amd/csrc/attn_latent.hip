@@ -116,7 +116,8 @@ template <typename T, int VEC>
 __global__ void __launch_bounds__(64)
 attn_latent_kernel(const T* __restrict__ qa, int qa_stride, T* __restrict__ out, int out_stride,
                    const T* __restrict__ cache, const int* __restrict__ block_tables, int bt_stride,
-                   const int* __restrict__ token_req, const int* __restrict__ positions, int H, int R, int E,
+                   const int* __restrict__ token_req, const int* __restrict__ positions,
+                   const int* __restrict__ row_list, int H, int R, int E,
                    int page_size, float scale, int n_split, float* __restrict__ part_acc, float* __restrict__ part_ml) {
     constexpr int HG = kLatentHeads, NP = kLatentMaxRank / 64 / VEC;   // pieces of VEC columns a lane owns
     extern __shared__ float qs[];                 // HG * (R + E) floats
@@ -124,7 +125,8 @@ attn_latent_kernel(const T* __restrict__ qa, int qa_stride, T* __restrict__ out,
     __shared__ long long krow[64];
     const int D = R + E, lane = threadIdx.x;
     const int n_groups = (H + HG - 1) / HG;
-    const int hg = blockIdx.x % n_groups, t = blockIdx.x / n_groups, split = blockIdx.y;
+    const int hg = blockIdx.x % n_groups, split = blockIdx.y;
+    const int t = row_list ? row_list[blockIdx.x / n_groups] : blockIdx.x / n_groups;
     const int h0 = hg * HG, nh = (H - h0 < HG) ? H - h0 : HG;
     const int pos = positions[t];
     const int* bt = block_tables + (size_t)token_req[t] * bt_stride;
@@ -248,8 +250,8 @@ attn_latent_kernel(const T* __restrict__ qa, int qa_stride, T* __restrict__ out,
 template <typename T>
 __global__ void __launch_bounds__(256)
 attn_latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml, int n_split, int H, int R,
-                         T* __restrict__ out, int out_stride) {
-    const int h = blockIdx.x % H, t = blockIdx.x / H;
+                         T* __restrict__ out, int out_stride, const int* __restrict__ row_list) {
+    const int h = blockIdx.x % H, t = row_list ? row_list[blockIdx.x / H] : blockIdx.x / H;
     const size_t p0 = ((size_t)t * H + h) * n_split;
     float m = -INFINITY;
     for (int s = 0; s < n_split; ++s) m = fmaxf(m, part_ml[2 * (p0 + s)]);
@@ -270,9 +272,9 @@ attn_latent_merge_kernel(const float* __restrict__ part_acc, const float* __rest
 }
 
 IC_EXPORT int ic_attn_latent(const void* qa, int qa_stride, void* out, int out_stride, int dtype, const void* cache,
-                             const int* block_tables, int bt_stride, const int* token_req, const int* positions, int T,
-                             int H, int R, int E, int page_size, float scale, int n_split, float* part_acc,
-                             float* part_ml, hipStream_t stream) {
+                             const int* block_tables, int bt_stride, const int* token_req, const int* positions,
+                             const int* row_list, int T, int H, int R, int E, int page_size, float scale, int n_split,
+                             float* part_acc, float* part_ml, hipStream_t stream) {
     if (T <= 0) return IC_OK;
     if (H <= 0 || R <= 0 || R > kLatentMaxRank || E < 0 || page_size <= 0 || n_split < 1 || n_split > 64) return IC_ERR_ARG;
     if (n_split > 1 && (!part_acc || !part_ml)) return IC_ERR_ARG;
@@ -284,8 +286,8 @@ IC_EXPORT int ic_attn_latent(const void* qa, int qa_stride, void* out, int out_s
     dim3 grid((unsigned)(T * n_groups), n_split), block(64);
 #define IC_LAT(TT, VV)                                                                                                 \
     hipLaunchKernelGGL((attn_latent_kernel<TT, VV>), grid, block, lds, stream, (const TT*)qa, qa_stride, (TT*)out,     \
-                       out_stride, (const TT*)cache, block_tables, bt_stride, token_req, positions, H, R, E, page_size, \
-                       scale, n_split, part_acc, part_ml)
+                       out_stride, (const TT*)cache, block_tables, bt_stride, token_req, positions, row_list, H, R, E,  \
+                       page_size, scale, n_split, part_acc, part_ml)
     if (dtype == IC_F32) {
         if (R % 4 == 0 && E % 4 == 0) IC_LAT(float, 4); else IC_LAT(float, 1);
     } else if (dtype == IC_BF16) {
@@ -296,10 +298,95 @@ IC_EXPORT int ic_attn_latent(const void* qa, int qa_stride, void* out, int out_s
     if (n_split > 1) {
         if (dtype == IC_F32)
             hipLaunchKernelGGL(attn_latent_merge_kernel<float>, dim3(T * H), dim3(256), 0, stream, part_acc, part_ml, n_split,
-                               H, R, (float*)out, out_stride);
+                               H, R, (float*)out, out_stride, row_list);
         else
             hipLaunchKernelGGL(attn_latent_merge_kernel<bf16>, dim3(T * H), dim3(256), 0, stream, part_acc, part_ml, n_split,
-                               H, R, (bf16*)out, out_stride);
+                               H, R, (bf16*)out, out_stride, row_list);
     }
+    return ic_launch_status();
+}
+
+// ---- prompt portions through matrix products -------------------------------------------------------------------------
+// For a portion of several tokens the walk is two products over all heads at once, rows = (token, head):
+// scores = Q' C^T and result = P C[:, :R].  The request's latent rows are gathered out of their pages into one
+// matrix (and its first R columns transposed, for the second product), the scores pass a masked softmax.
+
+// rows[j] = cache row of key j (j < L), zeros for L <= j < L_pad; rows_t[c, j] = rows[j, c] for c < R.
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_gather_kernel(const T* __restrict__ cache, const int* __restrict__ table, int page_size, int D, int R, int L,
+                     int L_pad, T* __restrict__ rows, T* __restrict__ rows_t) {
+    __shared__ T tile[64][65];
+    const int j0 = blockIdx.x * 64;
+    for (int jj = threadIdx.x / 64; jj < 64; jj += 4) {
+        const int j = j0 + jj;
+        if (j >= L_pad) break;
+        const T* src = j < L ? cache + ((long long)table[j / page_size] * page_size + j % page_size) * D : nullptr;
+        for (int c = threadIdx.x % 64; c < D; c += 64) rows[(size_t)j * D + c] = src ? src[c] : from_f32<T>(0.f);
+    }
+    __syncthreads();
+    for (int c0 = 0; c0 < R; c0 += 64) {
+        for (int jj = threadIdx.x / 64; jj < 64; jj += 4) {
+            const int j = j0 + jj, c = c0 + threadIdx.x % 64;
+            tile[jj][threadIdx.x % 64] = (j < L_pad && c < R) ? rows[(size_t)j * D + c] : from_f32<T>(0.f);
+        }
+        __syncthreads();
+        for (int cc = threadIdx.x / 64; cc < 64; cc += 4) {
+            const int c = c0 + cc, j = j0 + threadIdx.x % 64;
+            if (c < R && j < L_pad) rows_t[(size_t)c * L_pad + j] = tile[threadIdx.x % 64][cc];
+        }
+        __syncthreads();
+    }
+}
+
+IC_EXPORT int ic_latent_gather(const void* cache, int dtype, const int* table, int page_size, int D, int R, int L, int L_pad,
+                               void* rows, void* rows_t, hipStream_t stream) {
+    if (L <= 0) return IC_OK;
+    if (page_size <= 0 || D <= 0 || R <= 0 || R > D || L_pad < L) return IC_ERR_ARG;
+    dim3 grid((L_pad + 63) / 64), block(256);
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(latent_gather_kernel<float>, grid, block, 0, stream, (const float*)cache, table, page_size, D, R, L,
+                           L_pad, (float*)rows, (float*)rows_t);
+    else if (dtype == IC_BF16)
+        hipLaunchKernelGGL(latent_gather_kernel<bf16>, grid, block, 0, stream, (const bf16*)cache, table, page_size, D, R, L,
+                           L_pad, (bf16*)rows, (bf16*)rows_t);
+    else
+        return IC_ERR_UNSUPPORTED;
+    return ic_launch_status();
+}
+
+// Row m belongs to token m / H of the portion, which sees keys 0 .. first_limit + m / H.  p = softmax(scale * s) over
+// them, zero beyond (up to n_cols).  One block per row; the scores are float32.
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_softmax_kernel(const float* __restrict__ s, int lds, T* __restrict__ p, int ldp, int H, int n_cols, int first_limit,
+                      float scale) {
+    __shared__ float red[8];
+    const int m = blockIdx.x;
+    const int n = min(first_limit + m / H + 1, n_cols);
+    const float* row = s + (size_t)m * lds;
+    float mx = -INFINITY;
+    for (int j = threadIdx.x; j < n; j += blockDim.x) mx = fmaxf(mx, row[j]);
+    mx = block_max(mx, red) * scale;
+    float sum = 0.f;
+    for (int j = threadIdx.x; j < n; j += blockDim.x) sum += expf(row[j] * scale - mx);
+    const float inv = 1.0f / block_sum(sum, red);
+    T* out = p + (size_t)m * ldp;
+    for (int j = threadIdx.x; j < n_cols; j += blockDim.x)
+        out[j] = from_f32<T>(j < n ? expf(row[j] * scale - mx) * inv : 0.f);
+}
+
+IC_EXPORT int ic_latent_softmax(const float* s, int lds, void* p, int ldp, int dtype, int M, int H, int n_cols,
+                                int first_limit, float scale, hipStream_t stream) {
+    if (M <= 0) return IC_OK;
+    if (H <= 0 || n_cols <= 0 || first_limit < 0 || scale <= 0.f) return IC_ERR_ARG;
+    if (dtype == IC_F32)
+        hipLaunchKernelGGL(latent_softmax_kernel<float>, dim3(M), dim3(256), 0, stream, s, lds, (float*)p, ldp, H, n_cols,
+                           first_limit, scale);
+    else if (dtype == IC_BF16)
+        hipLaunchKernelGGL(latent_softmax_kernel<bf16>, dim3(M), dim3(256), 0, stream, s, lds, (bf16*)p, ldp, H, n_cols,
+                           first_limit, scale);
+    else
+        return IC_ERR_UNSUPPORTED;
     return ic_launch_status();
 }

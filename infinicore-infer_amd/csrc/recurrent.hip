@@ -97,45 +97,96 @@ IC_EXPORT int ic_causal_conv(const void* xin, int xin_stride, int dtype, const f
 // gate) and the same + bw (input gate), biases laid out alike.  With r, i their sigmoids:
 //     log a = decay[c] * r,  S <- exp(log a) S + sqrt(1 - exp(2 log a)) * i * u,  out = S * gelu_tanh(yb + y_bias).
 // decay[c] = -8 softplus(lam[c]), made once when the weights are loaded.
+//
+// Both recurrences of this file are linear in the state, S_end = A S_begin + S_local, so a long portion is cut into
+// chunks that run side by side: pass 1 (mode 1) runs every chunk from a zero state and leaves (S_local, A); a small
+// kernel walks a request's chunks in order and replaces S_local by the state the chunk really starts from (and
+// writes the request's new state); pass 2 (mode 2) runs every chunk again from there and writes the results.
+// mode 0 is the single pass from and to the request's state (few tokens).
 template <typename T>
 __global__ void __launch_bounds__(128)
 rglru_scan_kernel(const float* __restrict__ gates, const float* __restrict__ gate_bias, const float* __restrict__ u,
                   const T* __restrict__ yb, int yb_stride, const float* __restrict__ y_bias,
                   const float* __restrict__ decay, int width, int bw, T* __restrict__ out,
                   float* __restrict__ state, long long state_stride, const int* __restrict__ req_start,
-                  const int* __restrict__ state_slots) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+                  const int* __restrict__ state_slots, int mode, int chunk_len, int max_chunks,
+                  float* __restrict__ scr_s, float* __restrict__ scr_a) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y, ck = blockIdx.z;
     if (c >= width) return;
+    const int req_end = req_start[r + 1];
+    const int begin = req_start[r] + (mode ? ck * chunk_len : 0);
+    const int end = mode ? min(req_end, begin + chunk_len) : req_end;
+    if (begin >= req_end) return;
     const int g0 = (c / bw) * 2 * bw + c % bw;
     const float br = gate_bias[g0], bi = gate_bias[g0 + bw], dc = decay[c], yb0 = y_bias ? y_bias[c] : 0.f;
     float* st = state + (long long)state_slots[r] * state_stride;
-    float S = st[c];
-    const int end = req_start[r + 1];
-    for (int t = req_start[r]; t < end; ++t) {
+    const size_t si = ((size_t)r * max_chunks + ck) * width + c;
+    float S = mode == 0 ? st[c] : mode == 2 ? scr_s[si] : 0.f;
+    float a_total = 1.f;
+#pragma unroll 4
+    for (int t = begin; t < end; ++t) {
         const float* g = gates + (size_t)t * 2 * width;
         const float rg = sigmoid_f(g[g0] + br), ig = sigmoid_f(g[g0 + bw] + bi);
         const float la = dc * rg;
-        S = expf(la) * S + sqrtf(-expm1f(2.0f * la)) * ig * u[(size_t)t * width + c];
-        out[(size_t)t * width + c] = from_f32<T>(S * gelu_tanh_f(to_f32(yb[(size_t)t * yb_stride + c]) + yb0));
+        const float a = expf(la);
+        S = a * S + sqrtf(-expm1f(2.0f * la)) * ig * u[(size_t)t * width + c];
+        a_total *= a;
+        if (mode != 1)
+            out[(size_t)t * width + c] = from_f32<T>(S * gelu_tanh_f(to_f32(yb[(size_t)t * yb_stride + c]) + yb0));
     }
-    st[c] = S;
+    if (mode == 0) st[c] = S;
+    if (mode == 1) { scr_s[si] = S; scr_a[si] = a_total; }
+}
+
+// scr_s[r, k, e] <- the state chunk k of request r starts from; state <- the state after the last chunk.
+// `per`: state elements per factor (scr_a holds one factor per `per` elements: per channel, or per head).
+__global__ void __launch_bounds__(256)
+chunk_states_kernel(float* __restrict__ scr_s, const float* __restrict__ scr_a, int n_state, int per, int chunk_len,
+                    int max_chunks, float* __restrict__ state, long long state_stride,
+                    const int* __restrict__ req_start, const int* __restrict__ state_slots) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+    if (e >= n_state) return;
+    const int n = req_start[r + 1] - req_start[r];
+    const int chunks = (n + chunk_len - 1) / chunk_len;
+    float* st = state + (long long)state_slots[r] * state_stride;
+    float S = st[e];
+    for (int k = 0; k < chunks; ++k) {
+        const size_t i = ((size_t)r * max_chunks + k) * n_state + e;
+        const float local = scr_s[i];
+        scr_s[i] = S;
+        S = scr_a[((size_t)r * max_chunks + k) * (n_state / per) + e / per] * S + local;
+    }
+    st[e] = S;
 }
 
 IC_EXPORT int ic_rglru_scan(const float* gates, const float* gate_bias, const float* u, const void* yb, int yb_stride,
                             int dtype, const float* y_bias, const float* decay, int width, int bw, void* out,
                             float* state, long long state_stride, const int* req_start, const int* state_slots, int R,
-                            hipStream_t stream) {
+                            int chunk_len, int max_chunks, float* scr_s, float* scr_a, hipStream_t stream) {
     if (R <= 0) return IC_OK;
     if (width <= 0 || bw <= 0 || width % bw || !state) return IC_ERR_ARG;
-    dim3 grid((width + 127) / 128, R), block(128);
-    if (dtype == IC_F32)
-        hipLaunchKernelGGL(rglru_scan_kernel<float>, grid, block, 0, stream, gates, gate_bias, u, (const float*)yb, yb_stride,
-                           y_bias, decay, width, bw, (float*)out, state, state_stride, req_start, state_slots);
-    else if (dtype == IC_BF16)
-        hipLaunchKernelGGL(rglru_scan_kernel<bf16>, grid, block, 0, stream, gates, gate_bias, u, (const bf16*)yb, yb_stride,
-                           y_bias, decay, width, bw, (bf16*)out, state, state_stride, req_start, state_slots);
-    else
-        return IC_ERR_UNSUPPORTED;
+    const bool chunked = chunk_len > 0 && max_chunks > 1;
+    if (chunked && (!scr_s || !scr_a || max_chunks > 65535)) return IC_ERR_ARG;
+    dim3 block(128);
+    for (int pass = 0; pass < (chunked ? 3 : 1); ++pass) {
+        const int mode = chunked ? (pass == 0 ? 1 : 2) : 0;
+        if (chunked && pass == 1) {
+            hipLaunchKernelGGL(chunk_states_kernel, dim3((width + 255) / 256, R), dim3(256), 0, stream, scr_s, scr_a, width, 1,
+                               chunk_len, max_chunks, state, state_stride, req_start, state_slots);
+            continue;
+        }
+        dim3 grid((width + 127) / 128, R, chunked ? max_chunks : 1);
+        if (dtype == IC_F32)
+            hipLaunchKernelGGL(rglru_scan_kernel<float>, grid, block, 0, stream, gates, gate_bias, u, (const float*)yb, yb_stride,
+                               y_bias, decay, width, bw, (float*)out, state, state_stride, req_start, state_slots, mode,
+                               chunk_len, max_chunks, scr_s, scr_a);
+        else if (dtype == IC_BF16)
+            hipLaunchKernelGGL(rglru_scan_kernel<bf16>, grid, block, 0, stream, gates, gate_bias, u, (const bf16*)yb, yb_stride,
+                               y_bias, decay, width, bw, (bf16*)out, state, state_stride, req_start, state_slots, mode,
+                               chunk_len, max_chunks, scr_s, scr_a);
+        else
+            return IC_ERR_UNSUPPORTED;
+    }
     return ic_launch_status();
 }
 
@@ -143,76 +194,160 @@ IC_EXPORT int ic_rglru_scan(const float* gates, const float* gate_bias, const fl
 // xbc [T, inner + 2 G N] float32 holds x (heads x P), then B (G x N), then C (G x N) of every token.  Per head h
 // with group g = h / (heads / G), dt = softplus(dt_raw + dt_bias[h]):
 //     S <- exp(neg_a[h] dt) S + dt B_g x_h^T   (S is N x P),   y_h = S^T C_g + D[h] x_h.
-// One block per (head, request); the state stays in LDS while the block walks the request's tokens.
-template <typename T>
+// One block per (head, request, chunk).  Thread (grp, p) keeps column p of a run of NI rows of S in registers;
+// a token's B, C and x pass through LDS, the next token's are loaded while this one is computed.
+template <typename T, int NI>
 __global__ void __launch_bounds__(256)
 ssm_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ dt_raw, int dt_stride,
                 const float* __restrict__ dt_bias, const float* __restrict__ neg_a, const float* __restrict__ Dw,
                 int heads, int P, int N, int G, float* __restrict__ y, float* __restrict__ state,
-                long long state_stride, const int* __restrict__ req_start, const int* __restrict__ state_slots) {
+                long long state_stride, const int* __restrict__ req_start, const int* __restrict__ state_slots,
+                int mode, int chunk_len, int max_chunks, float* __restrict__ scr_s, float* __restrict__ scr_a) {
     extern __shared__ float lds[];
-    const int h = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+    const int h = blockIdx.x, r = blockIdx.y, ck = blockIdx.z, tid = threadIdx.x;
+    const int req_end = req_start[r + 1];
+    const int begin = req_start[r] + (mode ? ck * chunk_len : 0);
+    const int end = mode ? min(req_end, begin + chunk_len) : req_end;
+    if (begin >= req_end) return;
     const int g = h / (heads / G), inner = heads * P, ch = inner + 2 * G * N;
-    const int ngrp = 256 / P;                    // P <= 256
-    float* S = lds;                              // N * P
-    float* Bs = S + (size_t)N * P;               // N
-    float* Cs = Bs + N;                          // N
-    float* xs = Cs + N;                          // P
-    float* part = xs + P;                        // ngrp * P
+    const int ngrp = 256 / P, ni = (N + ngrp - 1) / ngrp;       // P <= 256, ni <= NI
+    const int grp = tid / P, p = tid % P, n0 = grp * ni;
+    const bool active = grp < ngrp;
+    const int bufsz = 2 * N + P;                                 // B, C, x of one token; <= 1024
+    float* buf0 = lds;
+    float* buf1 = lds + bufsz;
+    float* part = lds + 2 * bufsz;                               // ngrp * P
     float* st = state + (long long)state_slots[r] * state_stride + (size_t)h * N * P;
-    for (int e = tid; e < N * P; e += 256) S[e] = st[e];
+    float* sc = scr_s + (((size_t)r * max_chunks + ck) * heads + h) * N * P;
+    float s[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int n = n0 + i;
+        const bool ok = active && i < ni && n < N;
+        s[i] = !ok ? 0.f : mode == 0 ? st[n * P + p] : mode == 2 ? sc[n * P + p] : 0.f;
+    }
     const float db = dt_bias[h], na = neg_a[h], dw = Dw[h];
-    const int grp = tid / P, p = tid % P;
-    const int end = req_start[r + 1];
-    __syncthreads();
-    for (int t = req_start[r]; t < end; ++t) {
-        const float* row = xbc + (size_t)t * ch;
-        for (int n = tid; n < N; n += 256) {
-            Bs[n] = row[inner + g * N + n];
-            Cs[n] = row[inner + G * N + g * N + n];
+    const int off_b = inner + g * N, off_c = inner + G * N + g * N, off_x = h * P;
+    auto src = [&](int e) { return e < N ? off_b + e : e < 2 * N ? off_c + (e - N) : off_x + (e - 2 * N); };
+    float pre[4];
+    {
+        const float* row = xbc + (size_t)begin * ch;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int e = tid + 256 * k;
+            if (e < bufsz) buf0[e] = row[src(e)];
         }
-        for (int q = tid; q < P; q += 256) xs[q] = row[h * P + q];
-        const float dt = softplus_f(to_f32(dt_raw[(size_t)t * dt_stride + h]) + db);
+    }
+    float dt_next = to_f32(dt_raw[(size_t)begin * dt_stride + h]);
+    float a_total = 1.f;
+    __syncthreads();
+    for (int t = begin; t < end; ++t) {
+        float* cur = ((t - begin) & 1) ? buf1 : buf0;
+        float* nxt = ((t - begin) & 1) ? buf0 : buf1;
+        const float dt = softplus_f(dt_next + db);
+        const bool more = t + 1 < end;
+        if (more) {
+            const float* row = xbc + (size_t)(t + 1) * ch;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int e = tid + 256 * k;
+                if (e < bufsz) pre[k] = row[src(e)];
+            }
+            dt_next = to_f32(dt_raw[(size_t)(t + 1) * dt_stride + h]);
+        }
         const float da = expf(na * dt);
-        __syncthreads();
-        if (grp < ngrp) {
+        a_total *= da;
+        const float* Bs = cur;
+        const float* Cs = cur + N;
+        const float* xs = cur + 2 * N;
+        if (active) {
             const float dx = dt * xs[p];
             float acc = 0.f;
-            for (int n = grp; n < N; n += ngrp) {
-                const float s = da * S[n * P + p] + Bs[n] * dx;
-                S[n * P + p] = s;
-                acc += s * Cs[n];
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int n = n0 + i;
+                if (i < ni && n < N) {
+                    s[i] = da * s[i] + Bs[n] * dx;
+                    acc += s[i] * Cs[n];
+                }
             }
-            part[grp * P + p] = acc;
+            if (mode != 1) part[grp * P + p] = acc;
         }
         __syncthreads();
-        if (tid < P) {
+        if (mode != 1 && tid < P) {
             float acc = dw * xs[tid];
             for (int q = 0; q < ngrp; ++q) acc += part[q * P + tid];
             y[(size_t)t * inner + h * P + tid] = acc;
         }
+        if (more) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int e = tid + 256 * k;
+                if (e < bufsz) nxt[e] = pre[k];
+            }
+        }
         __syncthreads();
     }
-    for (int e = tid; e < N * P; e += 256) st[e] = S[e];
+    if (mode == 2) return;
+    float* dst = mode == 0 ? st : sc;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int n = n0 + i;
+        if (active && i < ni && n < N) dst[n * P + p] = s[i];
+    }
+    if (mode == 1 && tid == 0) scr_a[((size_t)r * max_chunks + ck) * heads + h] = a_total;
+}
+
+template <typename T>
+static int ssm_launch(int ni, dim3 grid, size_t lds, hipStream_t stream, const float* xbc, const void* dt_raw, int dt_stride,
+                      const float* dt_bias, const float* neg_a, const float* Dw, int heads, int P, int N, int G, float* y,
+                      float* state, long long state_stride, const int* req_start, const int* state_slots, int mode,
+                      int chunk_len, int max_chunks, float* scr_s, float* scr_a) {
+#define IC_SSM(NI)                                                                                                      \
+    hipLaunchKernelGGL((ssm_scan_kernel<T, NI>), grid, dim3(256), lds, stream, xbc, (const T*)dt_raw, dt_stride, dt_bias, \
+                       neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots, mode, chunk_len,       \
+                       max_chunks, scr_s, scr_a)
+    if (ni <= 8) IC_SSM(8);
+    else if (ni <= 16) IC_SSM(16);
+    else if (ni <= 32) IC_SSM(32);
+    else if (ni <= 64) IC_SSM(64);
+    else if (ni <= 128) IC_SSM(128);
+    else return IC_ERR_TOO_LARGE;
+#undef IC_SSM
+    return IC_OK;
 }
 
 IC_EXPORT int ic_ssm_scan(const float* xbc, const void* dt_raw, int dt_stride, int dtype, const float* dt_bias,
                           const float* neg_a, const float* Dw, int heads, int P, int N, int G, float* y, float* state,
-                          long long state_stride, const int* req_start, const int* state_slots, int R,
-                          hipStream_t stream) {
+                          long long state_stride, const int* req_start, const int* state_slots, int R, int chunk_len,
+                          int max_chunks, float* scr_s, float* scr_a, hipStream_t stream) {
     if (R <= 0) return IC_OK;
     if (heads <= 0 || P <= 0 || P > 256 || N <= 0 || G <= 0 || heads % G || !state) return IC_ERR_ARG;
-    const size_t lds = ((size_t)N * P + 2 * N + P + (size_t)(256 / P) * P) * sizeof(float);
-    if (lds > 64 * 1024) return IC_ERR_TOO_LARGE;
-    dim3 grid(heads, R), block(256);
-    if (dtype == IC_F32)
-        hipLaunchKernelGGL(ssm_scan_kernel<float>, grid, block, lds, stream, xbc, (const float*)dt_raw, dt_stride, dt_bias,
-                           neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots);
-    else if (dtype == IC_BF16)
-        hipLaunchKernelGGL(ssm_scan_kernel<bf16>, grid, block, lds, stream, xbc, (const bf16*)dt_raw, dt_stride, dt_bias,
-                           neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots);
-    else
-        return IC_ERR_UNSUPPORTED;
+    if (2 * N + P > 1024) return IC_ERR_TOO_LARGE;
+    const bool chunked = chunk_len > 0 && max_chunks > 1;
+    if (chunked && (!scr_s || !scr_a || max_chunks > 65535)) return IC_ERR_ARG;
+    const int ngrp = 256 / P, ni = (N + ngrp - 1) / ngrp;
+    const size_t lds = ((size_t)2 * (2 * N + P) + (size_t)ngrp * P) * sizeof(float);
+    for (int pass = 0; pass < (chunked ? 3 : 1); ++pass) {
+        const int mode = chunked ? (pass == 0 ? 1 : 2) : 0;
+        if (chunked && pass == 1) {
+            const int n_state = heads * N * P;
+            hipLaunchKernelGGL(chunk_states_kernel, dim3((n_state + 255) / 256, R), dim3(256), 0, stream, scr_s, scr_a, n_state,
+                               N * P, chunk_len, max_chunks, state, state_stride, req_start, state_slots);
+            continue;
+        }
+        dim3 grid(heads, R, chunked ? max_chunks : 1);
+        int st;
+        if (dtype == IC_F32)
+            st = ssm_launch<float>(ni, grid, lds, stream, xbc, dt_raw, dt_stride, dt_bias, neg_a, Dw, heads, P, N, G, y, state,
+                                   state_stride, req_start, state_slots, mode, chunk_len, max_chunks, scr_s, scr_a);
+        else if (dtype == IC_BF16)
+            st = ssm_launch<bf16>(ni, grid, lds, stream, xbc, dt_raw, dt_stride, dt_bias, neg_a, Dw, heads, P, N, G, y, state,
+                                  state_stride, req_start, state_slots, mode, chunk_len, max_chunks, scr_s, scr_a);
+        else
+            return IC_ERR_UNSUPPORTED;
+        if (st != IC_OK) return st;
+    }
     return ic_launch_status();
 }
 

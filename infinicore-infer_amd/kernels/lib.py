@@ -122,13 +122,15 @@ _SIGNATURES = {
     "ic_embed_streams": [_P, _P, _P, _P, _I, _P, _I, _I, _I, _P, _P, _P, _P],
     "ic_hc_step": [_P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _F, _P, _I, _P],
     "ic_causal_conv": [_P, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _P, _LL, _P, _P, _P, _I, _I, _P],
-    "ic_rglru_scan": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _P, _P, _LL, _P, _P, _I, _P],
-    "ic_ssm_scan": [_P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _LL, _P, _P, _I, _P],
+    "ic_rglru_scan": [_P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _P, _P, _LL, _P, _P, _I, _I, _I, _P, _P, _P],
+    "ic_ssm_scan": [_P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _P, _P, _LL, _P, _P, _I, _I, _I, _P, _P, _P],
     "ic_gated_group_norm": [_P, _P, _I, _I, _P, _I, _I, _F, _P, _I, _P],
     "ic_blocked_product": [_P, _I, _I, _P, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P],
     "ic_latent_prep": [_P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P],
     "ic_latent_q_rotate": [_P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _I, _I, _P],
-    "ic_attn_latent": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
+    "ic_attn_latent": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
+    "ic_latent_gather": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P],
+    "ic_latent_softmax": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
     "ic_argmax_static_max_rows": [],

@@ -930,9 +930,24 @@ def causal_conv(xin, w, b, out, state, state_offset: int, token_req, req_start, 
     return out
 
 
+def _chunk_scratch(chunks, n_state: int, n_factors: int, n_requests: int, what: str):
+    """(chunk_len, max_chunks, scratch for states, scratch for factors) of a recurrence run in chunks side by side, or
+    zeros and None for the single pass.  ``chunks`` = (chunk_len, max_chunks, float32 states, float32 factors)."""
+    if not chunks or chunks[1] <= 1:
+        return 0, 1, None, None
+    chunk_len, max_chunks, scr_s, scr_a = chunks
+    _dev(scr_s, scr_a)
+    _need(chunk_len > 0 and scr_s.dtype == torch.float32 and scr_a.dtype == torch.float32
+          and scr_s.numel() >= n_requests * max_chunks * n_state and scr_a.numel() >= n_requests * max_chunks * n_factors,
+          what + ": scratch for the chunks too small")
+    return int(chunk_len), int(max_chunks), scr_s.data_ptr(), scr_a.data_ptr()
+
+
 def rglru_scan(gates, gate_bias, u, yb, y_bias, decay, block_width: int, out, state, state_offset: int, req_start,
-               state_slots, n_requests: int):
-    """The gated diagonal recurrence over every request's rows (see csrc/recurrent.hip); out = S * gelu_tanh(yb + y_bias)."""
+               state_slots, n_requests: int, chunks=None):
+    """The gated diagonal recurrence over every request's rows (see csrc/recurrent.hip); out = S * gelu_tanh(yb + y_bias).
+    ``chunks``: (chunk_len, max_chunks, scratch, scratch) to run every request's rows as chunks side by side (every
+    request must fit max_chunks chunks of chunk_len rows)."""
     _dev(gates, gate_bias, u, yb, y_bias, decay, out, state, req_start, state_slots)
     T, width = u.shape
     for v, shape in ((gates, (T, 2 * width)), (u, (T, width))):
@@ -947,12 +962,13 @@ def rglru_scan(gates, gate_bias, u, yb, y_bias, decay, block_width: int, out, st
     _need(state_offset + width <= stride, "rglru_scan: state too small")
     check(get_lib().ic_rglru_scan(gates.data_ptr(), gate_bias.data_ptr(), u.data_ptr(), yb.data_ptr(), yb.stride(0),
                                   dtype_code(yb.dtype), _ptr(y_bias), decay.data_ptr(), width, int(block_width), out.data_ptr(),
-                                  sp, stride, req_start.data_ptr(), state_slots.data_ptr(), n_requests, _stream()), "rglru_scan")
+                                  sp, stride, req_start.data_ptr(), state_slots.data_ptr(), n_requests,
+                                  *_chunk_scratch(chunks, width, width, n_requests, "rglru_scan"), _stream()), "rglru_scan")
     return out
 
 
 def ssm_scan(xbc, dt_raw, dt_bias, neg_a, d_skip, heads: int, head_dim: int, state_dim: int, groups: int, y, state,
-             state_offset: int, req_start, state_slots, n_requests: int):
+             state_offset: int, req_start, state_slots, n_requests: int, chunks=None):
     """The state-space recurrence over every request's rows (see csrc/recurrent.hip): y float32 [T, heads * head_dim]."""
     _dev(xbc, dt_raw, dt_bias, neg_a, d_skip, y, state, req_start, state_slots)
     T = xbc.shape[0]
@@ -968,7 +984,8 @@ def ssm_scan(xbc, dt_raw, dt_bias, neg_a, d_skip, heads: int, head_dim: int, sta
     _need(state_offset + inner * state_dim <= stride, "ssm_scan: state too small")
     check(get_lib().ic_ssm_scan(xbc.data_ptr(), dt_raw.data_ptr(), dt_raw.stride(0), dtype_code(dt_raw.dtype), dt_bias.data_ptr(),
                                 neg_a.data_ptr(), d_skip.data_ptr(), heads, head_dim, state_dim, groups, y.data_ptr(), sp, stride,
-                                req_start.data_ptr(), state_slots.data_ptr(), n_requests, _stream()), "ssm_scan")
+                                req_start.data_ptr(), state_slots.data_ptr(), n_requests,
+                                *_chunk_scratch(chunks, inner * state_dim, heads, n_requests, "ssm_scan"), _stream()), "ssm_scan")
     return y
 
 
@@ -1037,11 +1054,17 @@ LATENT_MAX_RANK = 512
 
 
 def attention_latent(qa, out, cache, block_tables, token_req, positions, heads: int, kv_rank: int, rot_dim: int,
-                     page_size: int, scale: float, n_split: int = 1, part_acc=None, part_ml=None):
+                     page_size: int, scale: float, n_split: int = 1, part_acc=None, part_ml=None, row_list=None, n_rows=None):
     """out[t, h, :kv_rank] = sum_j p_j c_j over the cached rows [c | k_rot] j <= positions[t] of the token's request,
-    p = softmax(scale * qa[t, h] . row_j): every head walks the same rows."""
-    _dev(qa, out, cache, block_tables, token_req, positions, part_acc, part_ml)
+    p = softmax(scale * qa[t, h] . row_j): every head walks the same rows.  ``row_list`` (int32, ``n_rows`` of them): the
+    rows t to compute; None: all."""
+    _dev(qa, out, cache, block_tables, token_req, positions, part_acc, part_ml, row_list)
     T = qa.shape[0]
+    n_launch = T
+    if row_list is not None:
+        _i32(row_list, "row_list")
+        n_launch = int(n_rows)
+        _need(0 <= n_launch <= row_list.numel(), "attention_latent: row list shorter than n_rows")
     D = kv_rank + rot_dim
     _need(tuple(qa.shape) == (T, heads * D) and qa.stride(1) == 1 and out.dtype == qa.dtype
           and tuple(out.shape) == (T, heads * kv_rank) and out.stride(1) == 1, "attention_latent: q / out")
@@ -1056,6 +1079,31 @@ def attention_latent(qa, out, cache, block_tables, token_req, positions, heads: 
               "attention_latent: scratch too small")
     check(get_lib().ic_attn_latent(qa.data_ptr(), qa.stride(0), out.data_ptr(), out.stride(0), dtype_code(qa.dtype),
                                    cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(),
-                                   positions.data_ptr(), T, heads, kv_rank, rot_dim, page_size, float(scale), int(n_split),
-                                   _ptr(part_acc), _ptr(part_ml), _stream()), "attention_latent")
+                                   positions.data_ptr(), _ptr(row_list), n_launch, heads, kv_rank, rot_dim, page_size,
+                                   float(scale), int(n_split), _ptr(part_acc), _ptr(part_ml), _stream()), "attention_latent")
     return out
+
+
+def latent_gather(cache, table_row, n_keys: int, n_padded: int, page_size: int, kv_rank: int, rows, rows_t):
+    """rows[j] = the cached row of key j of the request whose block-table row is ``table_row`` (zeros from n_keys to
+    n_padded); rows_t[c, j] = rows[j, c] for the first kv_rank columns."""
+    _dev(cache, table_row, rows, rows_t)
+    D = cache.shape[-1]
+    _need(table_row.dtype == torch.int32 and table_row.stride(-1) == 1 and table_row.numel() * page_size >= n_keys,
+          "latent_gather: block table")
+    _need(cache.is_contiguous() and cache.shape[1] == 1 and cache.shape[2] == page_size, "latent_gather: cache plane")
+    _need(rows.dtype == cache.dtype and rows_t.dtype == cache.dtype and tuple(rows.shape) == (n_padded, D) and rows.is_contiguous()
+          and tuple(rows_t.shape) == (kv_rank, n_padded) and rows_t.is_contiguous() and n_padded >= n_keys, "latent_gather: outputs")
+    check(get_lib().ic_latent_gather(cache.data_ptr(), dtype_code(cache.dtype), table_row.data_ptr(), page_size, D, kv_rank,
+                                     int(n_keys), int(n_padded), rows.data_ptr(), rows_t.data_ptr(), _stream()), "latent_gather")
+
+
+def latent_softmax(scores, probs, heads: int, first_limit: int, scale: float):
+    """probs[m] = softmax(scale * scores[m, :n]) with n = first_limit + m // heads + 1 visible keys, zeros beyond."""
+    _dev(scores, probs)
+    M, n_cols = scores.shape
+    _need(scores.dtype == torch.float32 and scores.stride(1) == 1 and tuple(probs.shape) == (M, n_cols) and probs.stride(1) == 1,
+          "latent_softmax: layout")
+    check(get_lib().ic_latent_softmax(scores.data_ptr(), scores.stride(0), probs.data_ptr(), probs.stride(0), dtype_code(probs.dtype),
+                                      M, heads, n_cols, int(first_limit), float(scale), _stream()), "latent_softmax")
+    return probs

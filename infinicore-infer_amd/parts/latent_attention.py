@@ -77,14 +77,57 @@ class LatentAttention(Mixer):
         self.w_uk_t = tensors[n + "uk"].view(H, self.dim, self.R).transpose(1, 2).contiguous()
         self.w_uv = tensors[n + "uv"].view(H, self.dv, self.R).contiguous()
 
-    def _key_splits(self, ctx, T) -> int:
-        """Ways to split the keys of a step of single tokens, so that few rows still fill the chip: a function of the
-        step's shape (rows, rounded key count) alone."""
-        if T != ctx.R or not ctx.max_context:
+    def portion_tile_rows(self):
+        return ops.attention_prefill_tile_rows()       # the step lists its single-token rows: they take the walk kernel
+
+    def _key_splits(self, ctx, n_rows) -> int:
+        """Ways to split the keys of single-token rows, so that few rows still fill the chip: a function of the step's
+        shape (such rows, rounded key count) alone."""
+        if not n_rows or not ctx.max_context:
             return 1
-        waves = T * ((self.H + 3) // 4)
+        waves = n_rows * ((self.H + 3) // 4)
         chunks = (int(ctx.max_context) + 63) // 64
         return max(1, min(32, chunks // 2, (2 * ctx.cu_count + waves - 1) // waves))
+
+    def _attend(self, qa, walked, ctx, cache):
+        """Single-token rows walk the cached rows (keys split so that few rows fill the chip); a portion of several
+        tokens takes two matrix products over all its (token, head) rows (bfloat16; float32 walks everything)."""
+        rt, T, H, R, E = self.runtime, qa.shape[0], self.H, self.R, self.E
+        by_products = rt.dtype == torch.bfloat16 and rt.attention_impl == "auto" and ctx.n_decode_rows < T and (ctx.n_decode_rows > 0 or ctx.n_prefill_tiles > 0)
+        if by_products:
+            rows, n_rows = (None if ctx.decode_rows_identity else ctx.decode_rows), ctx.n_decode_rows
+        else:
+            rows, n_rows = None, T
+        if n_rows:
+            n_split = self._key_splits(ctx, n_rows) if (by_products or T == ctx.R) else 1
+            part_acc = part_ml = None
+            if n_split > 1:
+                part_acc = ctx.ws.buffer("latent_part_acc", (T * H * n_split * R,), torch.float32)
+                part_ml = ctx.ws.buffer("latent_part_ml", (T * H * n_split * 2,), torch.float32)
+            ops.attention_latent(qa, walked, cache.k, cache.block_tables, ctx.token_req, ctx.positions, H, R, E, ctx.page_size,
+                                 self.scale, n_split, part_acc, part_ml, row_list=rows, n_rows=n_rows)
+        if not by_products:
+            return
+        from .linear import _library
+        D = R + E
+        for r, n in enumerate(ctx.req_len):
+            if n < 2:
+                continue
+            row0, pos0 = ctx.req_start[r], ctx.req_pos[r]
+            L = pos0 + n
+            L_pad = (L + 15) // 16 * 16
+            gathered = ctx.ws.buffer("latent_gathered", (L_pad, D), rt.dtype)
+            gathered_t = ctx.ws.buffer("latent_gathered_t", (R, L_pad), rt.dtype)
+            ops.latent_gather(cache.k, cache.block_tables[r], L, L_pad, ctx.page_size, R, gathered, gathered_t)
+            per = max(1, min(n, (32 << 20) // (H * L_pad)))          # tokens per pass: the scores of a pass stay under 128 MB
+            for q0 in range(0, n, per):
+                qn = min(per, n - q0)
+                cols = min(L_pad, (pos0 + q0 + qn + 15) // 16 * 16)     # keys beyond the pass's last token are not computed
+                scores = ctx.ws.buffer("latent_scores", (qn * H, cols), torch.float32)
+                _library(qa[row0 + q0:row0 + q0 + qn].view(qn * H, D), gathered[:cols], scores)
+                probs = ctx.ws.buffer("latent_probs", (qn * H, cols), rt.dtype)
+                ops.latent_softmax(scores, probs, H, pos0 + q0, self.scale)
+                _library(probs, gathered_t[:, :cols], walked[row0 + q0:row0 + q0 + qn].view(qn * H, R))
 
     def forward(self, h, ctx, cache):
         rt, T, H, R, E = self.runtime, h.shape[0], self.H, self.R, self.E
@@ -99,13 +142,7 @@ class LatentAttention(Mixer):
         ops.blocked_product(q.view(T, H, self.dim + E)[:, :, :self.dim], self.w_uk_t, qa.view(T, H, R + E)[:, :, :R])
         ops.latent_q_rotate(q, self.dim, E, R, H, self.freq, self.rot_dims, ctx.positions, qa)
         walked = ctx.ws.buffer("latent_walk", (T, H * R), rt.dtype)
-        n_split = self._key_splits(ctx, T)
-        part_acc = part_ml = None
-        if n_split > 1:
-            part_acc = ctx.ws.buffer("latent_part_acc", (T * H * n_split * R,), torch.float32)
-            part_ml = ctx.ws.buffer("latent_part_ml", (T * H * n_split * 2,), torch.float32)
-        ops.attention_latent(qa, walked, cache.k, cache.block_tables, ctx.token_req, ctx.positions, H, R, E, ctx.page_size,
-                             self.scale, n_split, part_acc, part_ml)
+        self._attend(qa, walked, ctx, cache)
         heads_out = ctx.ws.buffer("latent_heads", (T, H * self.dv), rt.dtype)
         gate = rows[:, self.Rq + R + E:].view(T, H, self.dv) if self.gate else None
         ops.blocked_product(walked.view(T, H, R), self.w_uv, heads_out.view(T, H, self.dv), gate=gate)

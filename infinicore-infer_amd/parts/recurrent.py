@@ -18,6 +18,25 @@ from .base import CacheNeed, Mixer, register_part
 from .linear import linear
 
 
+CHUNK_SCRATCH_BYTES = 256 << 20     # most scratch memory the chunks' states of one recurrence may take
+
+
+def chunk_plan(ctx, n_state: int, n_factors: int, name: str):
+    """How a step's recurrence is cut into chunks that run side by side: None for a step of few tokens per request
+    (one pass from and to the state), else (chunk_len, max_chunks, scratch, scratch) with up to 32 chunks of at least 32
+    tokens for the longest portion, fewer where the chunks' states would not fit the scratch memory."""
+    longest = max(ctx.req_len) if ctx.req_len else 1
+    if longest < 64:
+        return None
+    most = max(1, min(32, longest // 32, CHUNK_SCRATCH_BYTES // (4 * n_state * ctx.R)))
+    if most <= 1:
+        return None
+    chunk_len = (longest + most - 1) // most
+    max_chunks = (longest + chunk_len - 1) // chunk_len
+    return (chunk_len, max_chunks, ctx.ws.buffer(name + "_chunk_states", (ctx.R * max_chunks * n_state,), torch.float32),
+            ctx.ws.buffer(name + "_chunk_factors", (ctx.R * max_chunks * n_factors,), torch.float32))
+
+
 @register_part("mixer", "rglru")
 class GatedLinearRecurrence(Mixer):
     graph_safe = True
@@ -78,7 +97,8 @@ class GatedLinearRecurrence(Mixer):
         ops.blocked_product((u if u_c is None else u_c).view(T, self.blocks, self.bw), self.w_gate,
                             gates.view(T, self.blocks, 2 * self.bw))
         out = ctx.ws.buffer("rglru_out", (T, w), rt.dtype)
-        ops.rglru_scan(gates, self.b_gate, u, yx[:, :w], self.b_y, self.decay, self.bw, out, cache.state, 0, *lists)
+        ops.rglru_scan(gates, self.b_gate, u, yx[:, :w], self.b_y, self.decay, self.bw, out, cache.state, 0, *lists,
+                       chunks=chunk_plan(ctx, w, w, "rglru"))
         y = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)
         linear(out, self.w_o, y, rt.gemm_impl, ws=ctx.ws)
         return y
@@ -95,8 +115,8 @@ class StateSpaceMixer(Mixer):
             raise ValueError("mamba2: %d heads are not a multiple of %d groups" % (heads, groups))
         if not 0 < head_dim <= 256:
             raise ValueError("mamba2: a head's size must lie in 1..256 (got %d)" % head_dim)
-        if state_dim <= 0 or (state_dim * head_dim + 2 * state_dim + 2 * 256) * 4 > 64 * 1024:
-            raise ValueError("mamba2: a head's state of %d x %d does not fit the kernel's local memory" % (state_dim, head_dim))
+        if state_dim <= 0 or 2 * state_dim + head_dim > 1024 or -(-state_dim // (256 // head_dim)) > 128:
+            raise ValueError("mamba2: a head's state of %d x %d is beyond what the kernel keeps in registers" % (state_dim, head_dim))
         self.inner = heads * head_dim
         if norm_groups <= 0 or self.inner % norm_groups:
             raise ValueError("mamba2: %d columns are not a multiple of %d norm groups" % (self.inner, norm_groups))
@@ -142,7 +162,7 @@ class StateSpaceMixer(Mixer):
                         ctx.token_req, *lists, act="silu")
         y = ctx.ws.buffer("ssm_y", (T, inner), torch.float32)
         ops.ssm_scan(xbc, proj[:, inner + ch:], self.dt_bias, self.neg_a, self.d_skip, self.heads, self.P, self.N, self.G, y,
-                     cache.state, 0, *lists)
+                     cache.state, 0, *lists, chunks=chunk_plan(ctx, inner * self.N, self.heads, "ssm"))
         g = ctx.ws.buffer("ssm_gated", (T, inner), rt.dtype)
         ops.gated_group_norm(y, proj[:, :inner], self.norm_w, self.norm_groups, self.eps, g)
         out = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)
