@@ -246,6 +246,169 @@ attn_latent_kernel(const T* __restrict__ qa, int qa_stride, T* __restrict__ out,
     }
 }
 
+// ---- the same walk on the matrix cores (bfloat16) --------------------------------------------------------------------
+// One block per (token, group of up to 32 heads, split of the keys); the heads are the 32 "queries" of
+// v_mfma_f32_32x32x16_bf16.  A step of 32 keys is loaded once into LDS as padded rows.  Scores are computed
+// transposed, S^T = K Q^T (A = 32 key rows x 16 values out of LDS, B = the heads' queries, held in registers), so a
+// lane holds 16 keys of ONE head, its partner lane (l ^ 32) the other 16, and the probabilities are already the B
+// operand of O^T = V^T P^T, whose A operand (the first R values of the same LDS rows, transposed) comes out of LDS
+// through the transposing read.  Operand layout (lane l, h = l / 32): A[i = l % 32][k = 8h..8h+7],
+// B[k = 8h..8h+7][j = l % 32], D[i = 8(r / 4) + 4h + r % 4][j = l % 32] for the 16 accumulators r.
+// A key beyond the token's position is replaced by the position's own row when loaded, and masked.
+typedef __bf16 lat_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float lat_v16f __attribute__((ext_vector_type(16)));
+typedef float lat_v8f __attribute__((ext_vector_type(8)));
+typedef short lat_v4s __attribute__((ext_vector_type(4)));
+
+template <int R, int E>
+__global__ void __launch_bounds__(64 * (R >= 128 ? 4 : R / 32))
+attn_latent_mfma_kernel(const bf16* __restrict__ qa, int qa_stride, bf16* __restrict__ out, int out_stride,
+                        const bf16* __restrict__ cache, const int* __restrict__ block_tables, int bt_stride,
+                        const int* __restrict__ token_req, const int* __restrict__ positions,
+                        const int* __restrict__ row_list, int H, int page_size, float scale, int n_split,
+                        float* __restrict__ part_acc, float* __restrict__ part_ml) {
+    // The block's waves share a step's rows in LDS; each computes the (same) scores and owns ND / WAVES of the
+    // 32-column tiles of the result.
+    constexpr int D = R + E, NC = D / 16, ND = R / 32, PK = D + 8, PIECES = D / 8;
+    constexpr int WAVES = ND >= 4 ? 4 : ND, NDW = ND / WAVES, THREADS = 64 * WAVES;
+    constexpr int NL = (32 * PIECES + THREADS - 1) / THREADS;       // 16-byte pieces of a step a thread loads
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[32 * PK];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lq = lane & 31, half = lane >> 5;
+    const int n_groups = (H + 31) / 32;
+    const int hg = blockIdx.x % n_groups, split = blockIdx.y;
+    const int t = row_list ? row_list[blockIdx.x / n_groups] : blockIdx.x / n_groups;
+    const int head = hg * 32 + lq;
+    const bool row_ok = head < H;
+    const int pos = positions[t];
+    const int* bt = block_tables + (size_t)token_req[t] * bt_stride;
+
+    lat_bf16x8 qf[NC];
+    {
+        const bf16* qp = qa + (size_t)t * qa_stride + (size_t)(row_ok ? head : 0) * D + 8 * half;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            uint4 v = *reinterpret_cast<const uint4*>(qp + 16 * c);
+            if (!row_ok) v = uint4{0u, 0u, 0u, 0u};
+            qf[c] = __builtin_bit_cast(lat_bf16x8, v);
+        }
+    }
+    const int n_steps = pos / 32 + 1;
+    const int per = (n_steps + n_split - 1) / n_split;
+    const int s_lo = split * per, s_hi = (s_lo + per < n_steps) ? s_lo + per : n_steps;
+
+    lat_v16f oacc[NDW];
+#pragma unroll
+    for (int i = 0; i < NDW; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    float m = -INFINITY, l = 0.f;
+    const float scale_log2e = scale * 1.4426950408889634f;
+    const int vrow = 4 * half + ((lane & 15) >> 2);
+    const int vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+    for (int s = s_lo; s < s_hi; ++s) {
+        const int kb = 32 * s;
+        uint4 got[NL];
+#pragma unroll
+        for (int k = 0; k < NL; ++k) {                      // every load is in flight before the first is stored
+            const int e = threadIdx.x + THREADS * k;
+            if (e < 32 * PIECES) {
+                const int row = e / PIECES, piece = e % PIECES;
+                const int key = (kb + row < pos) ? kb + row : pos;
+                got[k] = *reinterpret_cast<const uint4*>(cache + ((long long)bt[key / page_size] * page_size + key % page_size) * D + piece * 8);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < NL; ++k) {
+            const int e = threadIdx.x + THREADS * k;
+            if (e < 32 * PIECES) *reinterpret_cast<uint4*>(Ks + (e / PIECES) * PK + (e % PIECES) * 8) = got[k];
+        }
+        __syncthreads();
+        lat_v16f sacc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const lat_bf16x8 a = *reinterpret_cast<const lat_bf16x8*>(Ks + lq * PK + 16 * c + 8 * half);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], sacc, 0, 0, 0);
+        }
+        if (kb + 31 > pos) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (kb + 8 * (r >> 2) + 4 * half + (r & 3) > pos) sacc[r] = -INFINITY;
+        }
+        float mloc = sacc[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mloc = fmaxf(mloc, sacc[r]);
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+        const float m_new = fmaxf(m, mloc);                     // finite: the step's first key is visible
+        const float mc = m_new * scale_log2e;
+        const float corr = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m * scale_log2e - mc);
+        float rs = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float p = __builtin_amdgcn_exp2f(fmaf(sacc[r], scale_log2e, -mc));
+            sacc[r] = p;
+            rs += p;
+        }
+        rs += __shfl_xor(rs, 32, kWave);
+        l = l * corr + rs;
+        m = m_new;
+#pragma unroll
+        for (int i = 0; i < NDW; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][r] *= corr;
+#pragma unroll
+        for (int kc = 0; kc < 2; ++kc) {
+            lat_v8f pf;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = sacc[8 * kc + e];
+            const lat_bf16x8 b = __builtin_convertvector(pf, lat_bf16x8);
+#pragma unroll
+            for (int dt = 0; dt < NDW; ++dt) {
+                const uint16_t* vp = Ks + (16 * kc + vrow) * PK + 32 * (wave * NDW + dt) + vcol;
+                const lat_v4s lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lat_v4s __attribute__((address_space(3)))*)vp);
+                const lat_v4s hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lat_v4s __attribute__((address_space(3)))*)(vp + 8 * PK));
+                const lat_bf16x8 a = __builtin_bit_cast(lat_bf16x8, __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
+                oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, oacc[dt], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+    if (!row_ok) return;
+    if (n_split == 1) {
+        const float inv = 1.0f / l;
+        bf16* op = out + (size_t)t * out_stride + (size_t)head * R + 32 * wave * NDW;
+#pragma unroll
+        for (int dt = 0; dt < NDW; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) op[32 * dt + 8 * (r >> 2) + 4 * half + (r & 3)] = __float2bfloat16(oacc[dt][r] * inv);
+    } else {
+        const size_t pi = ((size_t)t * H + head) * n_split + split;
+        if (half == 0 && wave == 0) { part_ml[2 * pi] = m * scale; part_ml[2 * pi + 1] = l; }
+#pragma unroll
+        for (int dt = 0; dt < NDW; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                part_acc[pi * R + 32 * (wave * NDW + dt) + 8 * (r >> 2) + 4 * half + (r & 3)] = oacc[dt][r];
+    }
+}
+
+template <int R, int E>
+static void latent_mfma_launch(dim3 grid, hipStream_t stream, const void* qa, int qa_stride, void* out, int out_stride,
+                               const void* cache, const int* block_tables, int bt_stride, const int* token_req,
+                               const int* positions, const int* row_list, int H, int page_size, float scale, int n_split,
+                               float* part_acc, float* part_ml) {
+    hipLaunchKernelGGL((attn_latent_mfma_kernel<R, E>), grid, dim3(64 * (R >= 128 ? 4 : R / 32)), 0, stream, (const bf16*)qa, qa_stride, (bf16*)out,
+                       out_stride, (const bf16*)cache, block_tables, bt_stride, token_req, positions, row_list, H, page_size,
+                       scale, n_split, part_acc, part_ml);
+}
+
+// Sizes the matrix-core walk is built for: the latent 64, 128, 256 or 512 wide, the rotated part 16, 32 or 64.
+IC_EXPORT int ic_attn_latent_on_matrix_cores(int dtype, int R, int E) {
+    return dtype == IC_BF16 && (R == 64 || R == 128 || R == 256 || R == 512) && (E == 16 || E == 32 || E == 64);
+}
+
 // Merge of the splits: one block per (token, head).
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -274,13 +437,29 @@ attn_latent_merge_kernel(const float* __restrict__ part_acc, const float* __rest
 IC_EXPORT int ic_attn_latent(const void* qa, int qa_stride, void* out, int out_stride, int dtype, const void* cache,
                              const int* block_tables, int bt_stride, const int* token_req, const int* positions,
                              const int* row_list, int T, int H, int R, int E, int page_size, float scale, int n_split,
-                             float* part_acc, float* part_ml, hipStream_t stream) {
+                             float* part_acc, float* part_ml, int force_vector, hipStream_t stream) {
     if (T <= 0) return IC_OK;
     if (H <= 0 || R <= 0 || R > kLatentMaxRank || E < 0 || page_size <= 0 || n_split < 1 || n_split > 64) return IC_ERR_ARG;
     if (n_split > 1 && (!part_acc || !part_ml)) return IC_ERR_ARG;
     const int D = R + E;
     const size_t lds = (size_t)kLatentHeads * D * sizeof(float);
     if (lds > 60 * 1024) return IC_ERR_TOO_LARGE;
+    if (ic_attn_latent_on_matrix_cores(dtype, R, E) && scale > 0.f && !force_vector) {
+        const int wide_groups = (H + 31) / 32;
+        if ((long long)T * wide_groups > 0x7fffffffLL) return IC_ERR_ARG;
+        dim3 wide((unsigned)(T * wide_groups), n_split);
+#define IC_LATM(RR, EE)                                                                                                  \
+    if (R == RR && E == EE)                                                                                              \
+        latent_mfma_launch<RR, EE>(wide, stream, qa, qa_stride, out, out_stride, cache, block_tables, bt_stride, token_req, \
+                                   positions, row_list, H, page_size, scale, n_split, part_acc, part_ml);
+        IC_LATM(64, 16) IC_LATM(64, 32) IC_LATM(64, 64) IC_LATM(128, 16) IC_LATM(128, 32) IC_LATM(128, 64)
+        IC_LATM(256, 16) IC_LATM(256, 32) IC_LATM(256, 64) IC_LATM(512, 16) IC_LATM(512, 32) IC_LATM(512, 64)
+#undef IC_LATM
+        if (n_split > 1)
+            hipLaunchKernelGGL(attn_latent_merge_kernel<bf16>, dim3(T * H), dim3(256), 0, stream, part_acc, part_ml, n_split, H,
+                               R, (bf16*)out, out_stride, row_list);
+        return ic_launch_status();
+    }
     const int n_groups = (H + kLatentHeads - 1) / kLatentHeads;
     if ((long long)T * n_groups > 0x7fffffffLL) return IC_ERR_ARG;
     dim3 grid((unsigned)(T * n_groups), n_split), block(64);

@@ -128,7 +128,8 @@ _SIGNATURES = {
     "ic_blocked_product": [_P, _I, _I, _P, _I, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _P],
     "ic_latent_prep": [_P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _P, _P, _P, _P, _I, _P],
     "ic_latent_q_rotate": [_P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _I, _I, _P],
-    "ic_attn_latent": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P],
+    "ic_attn_latent": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _P],
+    "ic_attn_latent_on_matrix_cores": [_I, _I, _I],
     "ic_latent_gather": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P],
     "ic_latent_softmax": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],

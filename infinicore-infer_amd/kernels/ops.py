@@ -1053,11 +1053,19 @@ def latent_q_rotate(q, dim: int, rot_dim: int, kv_rank: int, heads: int, freq, r
 LATENT_MAX_RANK = 512
 
 
+def attention_latent_on_matrix_cores(dtype, kv_rank: int, rot_dim: int) -> bool:
+    """True when ``attention_latent`` runs its matrix-core kernel for these sizes."""
+    code = _code_or_none(dtype)
+    return code is not None and bool(get_lib().ic_attn_latent_on_matrix_cores(code, kv_rank, rot_dim))
+
+
 def attention_latent(qa, out, cache, block_tables, token_req, positions, heads: int, kv_rank: int, rot_dim: int,
-                     page_size: int, scale: float, n_split: int = 1, part_acc=None, part_ml=None, row_list=None, n_rows=None):
+                     page_size: int, scale: float, n_split: int = 1, part_acc=None, part_ml=None, row_list=None, n_rows=None,
+                     vector_units: bool = False):
     """out[t, h, :kv_rank] = sum_j p_j c_j over the cached rows [c | k_rot] j <= positions[t] of the token's request,
     p = softmax(scale * qa[t, h] . row_j): every head walks the same rows.  ``row_list`` (int32, ``n_rows`` of them): the
-    rows t to compute; None: all."""
+    rows t to compute; None: all.  bfloat16 with a latent of 64..512 and a rotated part of 16..64 values runs on the
+    matrix cores unless ``vector_units`` asks for the general kernel."""
     _dev(qa, out, cache, block_tables, token_req, positions, part_acc, part_ml, row_list)
     T = qa.shape[0]
     n_launch = T
@@ -1080,7 +1088,8 @@ def attention_latent(qa, out, cache, block_tables, token_req, positions, heads: 
     check(get_lib().ic_attn_latent(qa.data_ptr(), qa.stride(0), out.data_ptr(), out.stride(0), dtype_code(qa.dtype),
                                    cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(),
                                    positions.data_ptr(), _ptr(row_list), n_launch, heads, kv_rank, rot_dim, page_size,
-                                   float(scale), int(n_split), _ptr(part_acc), _ptr(part_ml), _stream()), "attention_latent")
+                                   float(scale), int(n_split), _ptr(part_acc), _ptr(part_ml), int(bool(vector_units)), _stream()),
+          "attention_latent")
     return out
 
 

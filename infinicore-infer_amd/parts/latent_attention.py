@@ -85,9 +85,10 @@ class LatentAttention(Mixer):
         shape (such rows, rounded key count) alone."""
         if not n_rows or not ctx.max_context:
             return 1
-        waves = n_rows * ((self.H + 3) // 4)
-        chunks = (int(ctx.max_context) + 63) // 64
-        return max(1, min(32, chunks // 2, (2 * ctx.cu_count + waves - 1) // waves))
+        on_cores = ops.attention_latent_on_matrix_cores(self.runtime.dtype, self.R, self.E)
+        blocks = n_rows * ((self.H + 31) // 32 if on_cores else (self.H + 3) // 4)
+        steps = (int(ctx.max_context) + 31) // 32 if on_cores else (int(ctx.max_context) + 63) // 64
+        return max(1, min(32, steps // 2, (2 * ctx.cu_count + blocks - 1) // blocks))
 
     def _attend(self, qa, walked, ctx, cache):
         """Single-token rows walk the cached rows (keys split so that few rows fill the chip); a portion of several

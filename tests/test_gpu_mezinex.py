@@ -21,11 +21,11 @@ BF16_WORST, BF16_SOME, BF16_MEAN = 0.5, 5e-2, 1.5e-2
 DTYPES = [("float32", torch.float32, 5e-4), ("bfloat16", torch.bfloat16, BF16_WORST)]
 
 
-def _compare(got, ref, dtype, tol, what, steps=None):
+def _compare(got, ref, dtype, tol, what, steps=None, mean=BF16_MEAN):
     worst = H.compare(got, ref, tol, what, steps)
     if dtype == torch.bfloat16:
         errs = [float((row.double() - ref[rid][pos]).abs().max()) / float(ref[rid].abs().max()) for (rid, pos), row in got.items()]
-        assert sum(errs) / len(errs) <= BF16_MEAN, "%s: mean error %.3g" % (what, sum(errs) / len(errs))
+        assert sum(errs) / len(errs) <= mean, "%s: mean error %.3g" % (what, sum(errs) / len(errs))
         assert sum(e > BF16_SOME for e in errs) <= max(2, 0.05 * len(errs)), "%s: %d of %d positions off by more than %.3g" % (
             what, sum(e > BF16_SOME for e in errs), len(errs), BF16_SOME)
     return worst
@@ -439,7 +439,7 @@ def _paged(rows_by_req, page_size, D, dtype, seed):
     return plane.cuda(), bt.cuda()
 
 
-@pytest.mark.parametrize("R,E,Hn,page", [(64, 32, 6, 16), (40, 8, 3, 16), (22, 6, 2, 32), (128, 64, 9, 64), (512, 64, 4, 16)])
+@pytest.mark.parametrize("R,E,Hn,page", [(64, 32, 6, 16), (40, 8, 3, 16), (22, 6, 2, 32), (128, 64, 40, 64), (512, 64, 4, 16)])
 @pytest.mark.parametrize("dname,dtype,tol", DTYPES)
 def test_walk_over_the_latent_rows(R, E, Hn, page, dname, dtype, tol):
     """Queries at positions around page borders and steps of 64 keys, single tokens with their keys split several ways,
@@ -469,15 +469,28 @@ def test_walk_over_the_latent_rows(R, E, Hn, page, dname, dtype, tol):
         assert p[i % Hn, far] > 0.2
     qa = q.reshape(T, Hn * D).cuda()
     req, posd = _i32([c[0] for c in cases]), _i32([c[1] for c in cases])
-    for n_split in (1, 3, 16):
+    from infinicore_infer_amd.kernels.lib import get_lib
+    on_cores = bool(get_lib().ic_attn_latent_on_matrix_cores(1 if dtype == torch.bfloat16 else 0, R, E))
+    assert on_cores == (dtype == torch.bfloat16 and (R, E) in ((64, 32), (128, 64), (512, 64)))
+    for n_split, vector in [(1, False), (3, False), (16, False)] + ([(1, True), (5, True)] if on_cores else []):
         out = torch.zeros(T, Hn * R, dtype=dtype, device="cuda")
         acc = torch.empty(T * Hn * n_split * R, dtype=torch.float32, device="cuda")
         ml = torch.empty(T * Hn * n_split * 2, dtype=torch.float32, device="cuda")
-        ops.attention_latent(qa, out, plane, bt, req, posd, Hn, R, E, page, scale, n_split, acc, ml)
+        ops.attention_latent(qa, out, plane, bt, req, posd, Hn, R, E, page, scale, n_split, acc, ml, vector_units=vector)
         got = out.view(T, Hn, R).cpu().double()
         assert torch.isfinite(got).all()
         err = (got - want).abs().amax(dim=(1, 2)) / want.abs().max()
-        assert float(err.max()) <= (2e-5 if dtype == torch.float32 else 2e-2), (n_split, cases[int(err.argmax())], float(err.max()))
+        assert float(err.max()) <= (2e-5 if dtype == torch.float32 else 2e-2), (n_split, vector, cases[int(err.argmax())], float(err.max()))
+    # a list of rows: only those are computed
+    rows = _i32([3, 0, T - 1])
+    out = torch.zeros(T, Hn * R, dtype=dtype, device="cuda")
+    ops.attention_latent(qa, out, plane, bt, req, posd, Hn, R, E, page, scale, row_list=rows, n_rows=3)
+    got = out.view(T, Hn, R).cpu().double()
+    for i in range(T):
+        if i in (3, 0, T - 1):
+            assert float((got[i] - want[i]).abs().max()) <= (2e-5 if dtype == torch.float32 else 2e-2) * float(want.abs().max())
+        else:
+            assert float(got[i].abs().max()) == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -577,7 +590,7 @@ def _drawn_config(seed):
         elif kind == "mamba2":
             groups = rng.choice([1, 2, 3])
             heads = groups * rng.choice([1, 2])
-            vdim = rng.choice([4, 12, 32])
+            vdim = rng.choice([8, 12, 32])
             ng = rng.choice([g for g in (1, 2, 3, 4, 6) if (heads * vdim) % g == 0 and heads * vdim // g >= 8])     # (a norm over a handful of values is a sign function: it magnifies any rounding)
             layers.append(_mamba(heads, vdim, rng.choice([4, 9, 16, 40]), groups, ng, rng.choice([1, 2, 3, 4]), ff))
         else:
@@ -611,6 +624,6 @@ def test_drawn_configurations(tmp_path_factory, seed):
     for dname, dtype, tol in DTYPES:
         engine = Engine.from_dir(folder, dtype=dtype, max_tokens=max_tokens, page_size=16, max_requests=4)
         # (tiny groups before a norm: one position of a bfloat16 run may flip; the mean and the count of such positions bound it)
-        _compare(H.run_trace(engine, steps), ref, dtype, tol if dtype == torch.float32 else 1.5, "drawn %d %s" % (seed, dname), steps)
+        _compare(H.run_trace(engine, steps), ref, dtype, tol if dtype == torch.float32 else 1.5, "drawn %d %s" % (seed, dname), steps, mean=4e-2)
         engine.cache.check_invariants()
         assert not engine.cache.requests
