@@ -13,6 +13,21 @@
 
 constexpr int kHcMaxStreams = 8;
 
+// four consecutive values as floats
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16* p) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    return float4{bf16_bits_to_f32((uint16_t)(v.x & 0xffff)), bf16_bits_to_f32((uint16_t)(v.x >> 16)),
+                  bf16_bits_to_f32((uint16_t)(v.y & 0xffff)), bf16_bits_to_f32((uint16_t)(v.y >> 16))};
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16* p, float4 v) {
+    uint2 o;
+    o.x = (uint32_t)f32_to_bf16_bits(v.x) | ((uint32_t)f32_to_bf16_bits(v.y) << 16);
+    o.y = (uint32_t)f32_to_bf16_bits(v.z) | ((uint32_t)f32_to_bf16_bits(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = o;
+}
+
 __global__ void pair_rows_kernel(const int* __restrict__ tokens, const int* __restrict__ positions,
                                  const int* __restrict__ token_req, const int* __restrict__ state_slots,
                                  const int* __restrict__ prev_state, int* __restrict__ rows, int T, long long buckets,
@@ -51,10 +66,22 @@ embed_streams_kernel(const int* __restrict__ tokens, const int* __restrict__ row
     const int tok = tokens[t];
     const T* e = table + (size_t)tok * d;
     const T* p = pair ? pair + (size_t)rows[t] * d : nullptr;
-    for (int j = threadIdx.x; j < d; j += blockDim.x) {
-        float v = to_f32(e[j]);
-        if (p) v += to_f32(p[j]);
-        for (int s = 0; s < n_streams; ++s) out[((size_t)s * n_tokens + t) * d + j] = v;
+    if (d % 4 == 0) {
+#pragma unroll 4
+        for (int j = 4 * threadIdx.x; j < d; j += 4 * blockDim.x) {
+            float4 v = load4(e + j);
+            if (p) {
+                const float4 w = load4(p + j);
+                v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+            }
+            for (int s = 0; s < n_streams; ++s) store4(out + ((size_t)s * n_tokens + t) * d + j, v);
+        }
+    } else {
+        for (int j = threadIdx.x; j < d; j += blockDim.x) {
+            float v = to_f32(e[j]);
+            if (p) v += to_f32(p[j]);
+            for (int s = 0; s < n_streams; ++s) out[((size_t)s * n_tokens + t) * d + j] = v;
+        }
     }
     if (prev_state && threadIdx.x == 0) {
         const int r = token_req[t];
@@ -98,40 +125,77 @@ hc_step_kernel(float* __restrict__ x, int n_tokens, int d, const TY* __restrict_
         for (int q = 0; q < S; ++q) m[s * S + q] = y ? mix[s * S + q] : 0.f;
     }
     float ss = 0.f;
-    for (int j = threadIdx.x; j < d; j += blockDim.x) {
-        float xs[S];
+    const int width = (d % 4 == 0) ? 4 : 1;          // four columns per thread and round where rows allow 16-byte accesses
+#pragma unroll 2
+    for (int j0 = width * threadIdx.x; j0 < d; j0 += width * blockDim.x) {
+        float xs[S][4], yv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (width == 4) {
 #pragma unroll
-        for (int s = 0; s < S; ++s) xs[s] = x[((size_t)s * n_tokens + t) * d + j];
+            for (int s = 0; s < S; ++s) {
+                const float4 v = load4(x + ((size_t)s * n_tokens + t) * d + j0);
+                xs[s][0] = v.x; xs[s][1] = v.y; xs[s][2] = v.z; xs[s][3] = v.w;
+            }
+            if (y) {
+                const float4 v = load4(y + (size_t)t * d + j0);
+                yv[0] = v.x; yv[1] = v.y; yv[2] = v.z; yv[3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < S; ++s) xs[s][0] = x[((size_t)s * n_tokens + t) * d + j0];
+            if (y) yv[0] = to_f32(y[(size_t)t * d + j0]);
+        }
         if (y) {
-            const float yv = to_f32(y[(size_t)t * d + j]);
-            float nx[S];
 #pragma unroll
-            for (int q = 0; q < S; ++q) {
-                float a = 0.f;
+            for (int e = 0; e < 4; ++e) {
+                if (e >= width) break;
+                float nx[S];
 #pragma unroll
-                for (int s = 0; s < S; ++s) a += m[s * S + q] * xs[s];
-                nx[q] = a + ow[q] * yv;
+                for (int q = 0; q < S; ++q) {
+                    float a = 0.f;
+#pragma unroll
+                    for (int s = 0; s < S; ++s) a += m[s * S + q] * xs[s][e];
+                    nx[q] = a + ow[q] * yv[e];
+                }
+#pragma unroll
+                for (int q = 0; q < S; ++q) xs[q][e] = nx[q];
             }
 #pragma unroll
             for (int q = 0; q < S; ++q) {
-                xs[q] = nx[q];
-                x[((size_t)q * n_tokens + t) * d + j] = nx[q];
+                float* dst = x + ((size_t)q * n_tokens + t) * d + j0;
+                if (width == 4) store4(dst, float4{xs[q][0], xs[q][1], xs[q][2], xs[q][3]});
+                else dst[0] = xs[q][0];
             }
         }
         if (in_w) {
-            float u = 0.f;
 #pragma unroll
-            for (int s = 0; s < S; ++s) u += iw[s] * xs[s];
-            u_row[j] = u;
-            ss += u * u;
+            for (int e = 0; e < 4; ++e) {
+                if (e >= width) break;
+                float u = 0.f;
+#pragma unroll
+                for (int s = 0; s < S; ++s) u += iw[s] * xs[s][e];
+                u_row[j0 + e] = u;
+                ss += u * u;
+            }
         }
     }
     if (!in_w) return;
     float r = 1.f;
     if (norm_w) r = 1.0f / sqrtf(block_sum(ss, red) / (float)d + eps);
-    for (int j = threadIdx.x; j < d; j += blockDim.x) {     // a thread reads back what it wrote itself
-        const float u = u_row[j];
-        h[(size_t)t * d + j] = from_f32<TH>(norm_w ? u * r * norm_w[j] : u);
+    if (width == 4) {
+#pragma unroll 2
+        for (int j0 = 4 * threadIdx.x; j0 < d; j0 += 4 * blockDim.x) {     // a thread reads back what it wrote itself
+            float4 u = *reinterpret_cast<const float4*>(u_row + j0);
+            if (norm_w) {
+                const float4 w = load4(norm_w + j0);
+                u = float4{u.x * r * w.x, u.y * r * w.y, u.z * r * w.z, u.w * r * w.w};
+            }
+            store4(h + (size_t)t * d + j0, u);
+        }
+    } else {
+        for (int j = threadIdx.x; j < d; j += blockDim.x) {
+            const float u = u_row[j];
+            h[(size_t)t * d + j] = from_f32<TH>(norm_w ? u * r * norm_w[j] : u);
+        }
     }
 }
 

@@ -448,10 +448,63 @@ blocked_product_kernel(const T* __restrict__ A, int lda, int a_step, const T* __
     }
 }
 
+// Up to 8 rows: nothing is tiled, the weights stream through once.  Eight lanes share a column and read its
+// weight row 16 bytes a lane (one cache line a round); the rows of A wait in LDS as floats.
+template <typename T, typename TC, int MT>
+__global__ void __launch_bounds__(256)
+blocked_product_rows_kernel(const T* __restrict__ A, int lda, int a_step, const T* __restrict__ W, TC* __restrict__ C,
+                            int ldc, int c_step, const T* __restrict__ gate, int gate_stride, int M, int N, int K) {
+    constexpr int VEC = 16 / sizeof(T);
+    extern __shared__ float a_rows[];         // MT * K
+    const int b = blockIdx.y, n = blockIdx.x * 32 + threadIdx.x / 8, sub = threadIdx.x % 8;
+    for (int e = threadIdx.x; e < MT * K; e += 256) {
+        const int mm = e / K, k = e % K;
+        a_rows[e] = mm < M ? to_f32(A[(size_t)mm * lda + (size_t)b * a_step + k]) : 0.f;
+    }
+    __syncthreads();
+    float acc[MT];
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) acc[mm] = 0.f;
+    const T* wrow = W + ((size_t)b * N + (n < N ? n : 0)) * K;
+#pragma unroll 4
+    for (int ch = sub; ch < K / VEC; ch += 8) {
+        alignas(16) T wv[VEC];
+        *reinterpret_cast<uint4*>(wv) = load_stream16(wrow + ch * VEC);
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            const float wf = to_f32(wv[v]);
+#pragma unroll
+            for (int mm = 0; mm < MT; ++mm) acc[mm] += a_rows[mm * K + ch * VEC + v] * wf;
+        }
+    }
+#pragma unroll
+    for (int mm = 0; mm < MT; ++mm) {
+        float v = acc[mm];
+        v += __shfl_xor(v, 4, kWave);
+        v += __shfl_xor(v, 2, kWave);
+        v += __shfl_xor(v, 1, kWave);
+        if (sub == 0 && n < N && mm < M) {
+            if (gate) v *= sigmoid_f(to_f32(gate[(size_t)mm * gate_stride + (size_t)b * c_step + n]));
+            C[(size_t)mm * ldc + (size_t)b * c_step + n] = from_f32<TC>(v);
+        }
+    }
+}
+
 template <typename T, typename TC>
 static void blocked_product_launch(const void* A, int lda, int a_step, const void* W, void* C, int ldc, int c_step,
                                    const void* gate, int gate_stride, int M, int N, int K, int B, hipStream_t stream) {
-    if (M <= 16) {
+    constexpr int VEC = 16 / sizeof(T);
+    if (M <= 8 && K % VEC == 0 && (size_t)8 * K * sizeof(float) <= 48 * 1024 && ((uintptr_t)W % 16) == 0) {
+        dim3 grid((N + 31) / 32, B);
+#define IC_ROWS(MT)                                                                                                   \
+    hipLaunchKernelGGL((blocked_product_rows_kernel<T, TC, MT>), grid, dim3(256), (size_t)MT * K * sizeof(float), stream, \
+                       (const T*)A, lda, a_step, (const T*)W, (TC*)C, ldc, c_step, (const T*)gate, gate_stride, M, N, K)
+        if (M == 1) IC_ROWS(1); else if (M == 2) IC_ROWS(2); else if (M <= 4) IC_ROWS(4); else IC_ROWS(8);
+#undef IC_ROWS
+        return;
+    }
+    // 16-row tiles for few rows, and wherever 64-row tiles would be fewer blocks than the chip has compute units
+    if (M <= 16 || (long long)((N + 63) / 64) * ((M + 63) / 64) * B < 256) {
         dim3 grid((N + 63) / 64, (M + 15) / 16, B);
         hipLaunchKernelGGL((blocked_product_kernel<T, TC, 16>), grid, dim3(256), 0, stream, (const T*)A, lda, a_step,
                            (const T*)W, (TC*)C, ldc, c_step, (const T*)gate, gate_stride, M, N, K);
