@@ -272,7 +272,9 @@ attn_latent_mfma_kernel(const bf16* __restrict__ qa, int qa_stride, bf16* __rest
     constexpr int D = R + E, NC = D / 16, ND = R / 32, PK = D + 8, PIECES = D / 8;
     constexpr int WAVES = ND >= 4 ? 4 : ND, NDW = ND / WAVES, THREADS = 64 * WAVES;
     constexpr int NL = (32 * PIECES + THREADS - 1) / THREADS;       // 16-byte pieces of a step a thread loads
+    constexpr bool QLDS = NC > 20;         // long rows: the queries wait in LDS (in registers they would halve the waves a unit holds)
     __shared__ __attribute__((aligned(16))) uint16_t Ks[32 * PK];
+    __shared__ __attribute__((aligned(16))) uint16_t Qs[QLDS ? 32 * PK : 8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, lq = lane & 31, half = lane >> 5;
     const int n_groups = (H + 31) / 32;
     const int hg = blockIdx.x % n_groups, split = blockIdx.y;
@@ -282,14 +284,16 @@ attn_latent_mfma_kernel(const bf16* __restrict__ qa, int qa_stride, bf16* __rest
     const int pos = positions[t];
     const int* bt = block_tables + (size_t)token_req[t] * bt_stride;
 
-    lat_bf16x8 qf[NC];
+    lat_bf16x8 qf[QLDS ? 1 : NC];
     {
         const bf16* qp = qa + (size_t)t * qa_stride + (size_t)(row_ok ? head : 0) * D + 8 * half;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
+            if (QLDS && c % WAVES != wave) continue;          // the waves write the queries' pieces in turn
             uint4 v = *reinterpret_cast<const uint4*>(qp + 16 * c);
             if (!row_ok) v = uint4{0u, 0u, 0u, 0u};
-            qf[c] = __builtin_bit_cast(lat_bf16x8, v);
+            if (QLDS) *reinterpret_cast<uint4*>(Qs + lq * PK + 16 * c + 8 * half) = v;
+            else qf[c] = __builtin_bit_cast(lat_bf16x8, v);
         }
     }
     const int n_steps = pos / 32 + 1;
@@ -306,11 +310,12 @@ attn_latent_mfma_kernel(const bf16* __restrict__ qa, int qa_stride, bf16* __rest
     const int vrow = 4 * half + ((lane & 15) >> 2);
     const int vcol = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-    for (int s = s_lo; s < s_hi; ++s) {
-        const int kb = 32 * s;
-        uint4 got[NL];
+    // A step's rows are asked for one step ahead: while this step is computed out of LDS the next one's loads are in flight.
+    uint4 got[NL];
+    auto fetch = [&](int step) {
+        const int kb = 32 * step;
 #pragma unroll
-        for (int k = 0; k < NL; ++k) {                      // every load is in flight before the first is stored
+        for (int k = 0; k < NL; ++k) {
             const int e = threadIdx.x + THREADS * k;
             if (e < 32 * PIECES) {
                 const int row = e / PIECES, piece = e % PIECES;
@@ -318,19 +323,25 @@ attn_latent_mfma_kernel(const bf16* __restrict__ qa, int qa_stride, bf16* __rest
                 got[k] = *reinterpret_cast<const uint4*>(cache + ((long long)bt[key / page_size] * page_size + key % page_size) * D + piece * 8);
             }
         }
+    };
+    if (s_lo < s_hi) fetch(s_lo);
+    for (int s = s_lo; s < s_hi; ++s) {
+        const int kb = 32 * s;
 #pragma unroll
         for (int k = 0; k < NL; ++k) {
             const int e = threadIdx.x + THREADS * k;
             if (e < 32 * PIECES) *reinterpret_cast<uint4*>(Ks + (e / PIECES) * PK + (e % PIECES) * 8) = got[k];
         }
         __syncthreads();
+        if (s + 1 < s_hi) fetch(s + 1);
         lat_v16f sacc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const lat_bf16x8 a = *reinterpret_cast<const lat_bf16x8*>(Ks + lq * PK + 16 * c + 8 * half);
-            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], sacc, 0, 0, 0);
+            const lat_bf16x8 q = QLDS ? *reinterpret_cast<const lat_bf16x8*>(Qs + lq * PK + 16 * c + 8 * half) : qf[c];
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q, sacc, 0, 0, 0);
         }
         if (kb + 31 > pos) {
 #pragma unroll
