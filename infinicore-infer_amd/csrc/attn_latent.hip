@@ -506,26 +506,29 @@ template <typename T>
 __global__ void __launch_bounds__(256)
 latent_gather_kernel(const T* __restrict__ cache, const int* __restrict__ table, int page_size, int D, int R, int L,
                      int L_pad, T* __restrict__ rows, T* __restrict__ rows_t) {
+    // blockIdx.y == 0: 64 keys' rows as they are; blockIdx.y = 1 + i: columns 64 i .. 64 i + 63 of the same keys, transposed
     __shared__ T tile[64][65];
-    const int j0 = blockIdx.x * 64;
-    for (int jj = threadIdx.x / 64; jj < 64; jj += 4) {
-        const int j = j0 + jj;
-        if (j >= L_pad) break;
-        const T* src = j < L ? cache + ((long long)table[j / page_size] * page_size + j % page_size) * D : nullptr;
-        for (int c = threadIdx.x % 64; c < D; c += 64) rows[(size_t)j * D + c] = src ? src[c] : from_f32<T>(0.f);
+    const int j0 = blockIdx.x * 64, lane = threadIdx.x % 64, w = threadIdx.x / 64;
+    if (blockIdx.y == 0) {
+        for (int jj = w; jj < 64; jj += 4) {
+            const int j = j0 + jj;
+            if (j >= L_pad) break;
+            const T* src = j < L ? cache + ((long long)table[j / page_size] * page_size + j % page_size) * D : nullptr;
+            for (int c = lane; c < D; c += 64) rows[(size_t)j * D + c] = src ? src[c] : from_f32<T>(0.f);
+        }
+        return;
+    }
+    const int c0 = 64 * (blockIdx.y - 1);
+    for (int jj = w; jj < 64; jj += 4) {
+        const int j = j0 + jj, c = c0 + lane;
+        T v = from_f32<T>(0.f);
+        if (j < L && c < R) v = cache[((long long)table[j / page_size] * page_size + j % page_size) * D + c];
+        tile[jj][lane] = v;
     }
     __syncthreads();
-    for (int c0 = 0; c0 < R; c0 += 64) {
-        for (int jj = threadIdx.x / 64; jj < 64; jj += 4) {
-            const int j = j0 + jj, c = c0 + threadIdx.x % 64;
-            tile[jj][threadIdx.x % 64] = (j < L_pad && c < R) ? rows[(size_t)j * D + c] : from_f32<T>(0.f);
-        }
-        __syncthreads();
-        for (int cc = threadIdx.x / 64; cc < 64; cc += 4) {
-            const int c = c0 + cc, j = j0 + threadIdx.x % 64;
-            if (c < R && j < L_pad) rows_t[(size_t)c * L_pad + j] = tile[threadIdx.x % 64][cc];
-        }
-        __syncthreads();
+    for (int cc = w; cc < 64; cc += 4) {
+        const int c = c0 + cc, j = j0 + lane;
+        if (c < R && j < L_pad) rows_t[(size_t)c * L_pad + j] = tile[lane][cc];
     }
 }
 
@@ -533,7 +536,7 @@ IC_EXPORT int ic_latent_gather(const void* cache, int dtype, const int* table, i
                                void* rows, void* rows_t, hipStream_t stream) {
     if (L <= 0) return IC_OK;
     if (page_size <= 0 || D <= 0 || R <= 0 || R > D || L_pad < L) return IC_ERR_ARG;
-    dim3 grid((L_pad + 63) / 64), block(256);
+    dim3 grid((L_pad + 63) / 64, 1 + (R + 63) / 64), block(256);
     if (dtype == IC_F32)
         hipLaunchKernelGGL(latent_gather_kernel<float>, grid, block, 0, stream, (const float*)cache, table, page_size, D, R, L,
                            L_pad, (float*)rows, (float*)rows_t);
@@ -555,13 +558,37 @@ latent_softmax_kernel(const float* __restrict__ s, int lds, T* __restrict__ p, i
     const int m = blockIdx.x;
     const int n = min(first_limit + m / H + 1, n_cols);
     const float* row = s + (size_t)m * lds;
+    T* out = p + (size_t)m * ldp;
+    if (n_cols <= 16 * 256) {                 // the row is read once and waits in registers
+        float v[16];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const int j = threadIdx.x + 256 * k;
+            v[k] = j < n ? row[j] : -INFINITY;
+            mx = fmaxf(mx, v[k]);
+        }
+        mx = block_max(mx, red) * scale;
+        float sum = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            v[k] = expf(v[k] * scale - mx);       // exp(-inf) = 0 beyond the visible keys
+            sum += v[k];
+        }
+        const float inv = 1.0f / block_sum(sum, red);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const int j = threadIdx.x + 256 * k;
+            if (j < n_cols) out[j] = from_f32<T>(v[k] * inv);
+        }
+        return;
+    }
     float mx = -INFINITY;
     for (int j = threadIdx.x; j < n; j += blockDim.x) mx = fmaxf(mx, row[j]);
     mx = block_max(mx, red) * scale;
     float sum = 0.f;
     for (int j = threadIdx.x; j < n; j += blockDim.x) sum += expf(row[j] * scale - mx);
     const float inv = 1.0f / block_sum(sum, red);
-    T* out = p + (size_t)m * ldp;
     for (int j = threadIdx.x; j < n_cols; j += blockDim.x)
         out[j] = from_f32<T>(j < n ? expf(row[j] * scale - mx) * inv : 0.f);
 }

@@ -496,6 +496,33 @@ def test_walk_over_the_latent_rows(R, E, Hn, page, dname, dtype, tol):
             assert float(got[i].abs().max()) == 0
 
 
+@pytest.mark.parametrize("R,E,page,L,first", [(64, 32, 16, 150, 0), (40, 8, 32, 70, 33), (128, 64, 64, 5000, 4990), (24, 8, 16, 17, 3)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gathered_rows_and_the_masked_softmax_of_prompt_portions(R, E, page, L, first, dtype):
+    """The pieces of the walk by matrix products: a request's rows out of shuffled pages (and their first R columns
+    transposed, zero beyond the last key), and the softmax whose row m sees the keys up to first + m // heads."""
+    from infinicore_infer_amd.kernels import ops
+    D, Hn = R + E, 3
+    g = torch.Generator().manual_seed(L)
+    rows = [torch.randn(7, D, generator=g), torch.randn(L, D, generator=g).to(dtype).float()]
+    plane, bt = _paged(rows, page, D, dtype, seed=L)
+    L_pad = (L + 15) // 16 * 16
+    got = torch.full((L_pad, D), float("nan"), dtype=dtype, device="cuda")
+    got_t = torch.full((R, L_pad), float("nan"), dtype=dtype, device="cuda")
+    ops.latent_gather(plane, bt[1], L, L_pad, page, R, got, got_t)
+    assert torch.equal(got[:L].float().cpu(), rows[1]) and float(got[L:].float().abs().sum()) == 0
+    assert torch.equal(got_t.float().cpu(), got[:, :R].float().cpu().T)
+    n = L - first                      # the portion's tokens: positions first .. L - 1
+    scores = torch.randn(n * Hn, L_pad, generator=g) * 3
+    probs = torch.full((n * Hn, L_pad), float("nan"), dtype=dtype, device="cuda")
+    ops.latent_softmax(scores.cuda(), probs, Hn, first, 0.37)
+    want = torch.zeros(n * Hn, L_pad, dtype=torch.float64)
+    for m in range(n * Hn):
+        k = first + m // Hn + 1
+        want[m, :k] = torch.softmax(scores[m, :k].double() * 0.37, dim=-1)
+    assert torch.allclose(probs.float().cpu().double(), want, atol=1e-6 if dtype == torch.float32 else 4e-3)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_latent_norms_rotation_and_cache_write(dtype):
     """The query latent's norm, the key latent's norm and the rotated key part at positions up to 60,000, written to the
