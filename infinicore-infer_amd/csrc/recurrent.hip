@@ -490,6 +490,57 @@ blocked_product_rows_kernel(const T* __restrict__ A, int lda, int a_step, const 
     }
 }
 
+// More than 8 rows in bfloat16 on the matrix cores: a wave owns 32 rows x 32 columns and computes them transposed,
+// C^T = W A^T with v_mfma_f32_32x32x16_bf16, so that both operands are 16 bytes a lane of a row as it lies in memory
+// (A operand: weight row l % 32, values 8h..8h+7 of the step; B operand: row l % 32 of A, the same values) and nothing
+// passes LDS.  Accumulator r of a lane is column 8(r / 4) + 4h + r % 4 of its row.
+typedef __bf16 bp_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float bp_v16f __attribute__((ext_vector_type(16)));
+
+template <typename TC>
+__global__ void __launch_bounds__(256)
+blocked_product_mfma_kernel(const bf16* __restrict__ A, int lda, int a_step, const bf16* __restrict__ W, TC* __restrict__ C,
+                            int ldc, int c_step, const bf16* __restrict__ gate, int gate_stride, int M, int N, int K) {
+    const int b = blockIdx.z, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lq = lane & 31, half = lane >> 5;
+    const int m0 = blockIdx.y * 64 + 32 * (wave >> 1), n0 = blockIdx.x * 64 + 32 * (wave & 1);
+    if (m0 >= M || n0 >= N) return;
+    const int m = m0 + lq, n = n0 + lq;
+    const bf16* ap = A + (size_t)(m < M ? m : M - 1) * lda + (size_t)b * a_step + 8 * half;
+    const bf16* wp = W + ((size_t)b * N + (n < N ? n : N - 1)) * K + 8 * half;
+    bp_v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    int k0 = 0;
+    for (; k0 + 64 <= K; k0 += 64) {              // four steps' loads in flight together
+        bp_bf16x8 wv[4], av[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            wv[i] = *reinterpret_cast<const bp_bf16x8*>(wp + k0 + 16 * i);
+            av[i] = *reinterpret_cast<const bp_bf16x8*>(ap + k0 + 16 * i);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv[i], av[i], acc, 0, 0, 0);
+    }
+    for (; k0 < K; k0 += 16) {
+        const bp_bf16x8 wv = *reinterpret_cast<const bp_bf16x8*>(wp + k0);
+        const bp_bf16x8 av = *reinterpret_cast<const bp_bf16x8*>(ap + k0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wv, av, acc, 0, 0, 0);
+    }
+    if (m >= M) return;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int nn = n0 + 8 * (r >> 2) + 4 * half + (r & 3);
+        if (nn < N) {
+            float v = acc[r];
+            if (gate) v *= sigmoid_f(to_f32(gate[(size_t)m * gate_stride + (size_t)b * c_step + nn]));
+            C[(size_t)m * ldc + (size_t)b * c_step + nn] = from_f32<TC>(v);
+        }
+    }
+}
+
+template <typename T> struct bp_is_bf16 { static constexpr bool value = false; };
+template <> struct bp_is_bf16<bf16> { static constexpr bool value = true; };
+
 template <typename T, typename TC>
 static void blocked_product_launch(const void* A, int lda, int a_step, const void* W, void* C, int ldc, int c_step,
                                    const void* gate, int gate_stride, int M, int N, int K, int B, hipStream_t stream) {
@@ -502,6 +553,14 @@ static void blocked_product_launch(const void* A, int lda, int a_step, const voi
         if (M == 1) IC_ROWS(1); else if (M == 2) IC_ROWS(2); else if (M <= 4) IC_ROWS(4); else IC_ROWS(8);
 #undef IC_ROWS
         return;
+    }
+    if constexpr (bp_is_bf16<T>::value) {
+        if (M > 8 && K % 16 == 0 && lda % 8 == 0 && a_step % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0) {
+            dim3 grid((N + 63) / 64, (M + 63) / 64, B);
+            hipLaunchKernelGGL((blocked_product_mfma_kernel<TC>), grid, dim3(256), 0, stream, (const bf16*)A, lda, a_step,
+                               (const bf16*)W, (TC*)C, ldc, c_step, (const bf16*)gate, gate_stride, M, N, K);
+            return;
+        }
     }
     // 16-row tiles for few rows, and wherever 64-row tiles would be fewer blocks than the chip has compute units
     if (M <= 16 || (long long)((N + 63) / 64) * ((M + 63) / 64) * B < 256) {

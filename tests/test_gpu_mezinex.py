@@ -400,7 +400,7 @@ def test_gate_and_norm_in_groups():
     assert torch.allclose(out.cpu().double(), want, atol=1e-5)
 
 
-@pytest.mark.parametrize("M,B,N,K", [(1, 3, 40, 24), (9, 2, 130, 70), (70, 4, 64, 16), (200, 1, 33, 129), (5, 2, 70, 64), (2, 3, 33, 40), (1, 3, 40, 21), (8, 40, 128, 512), (40, 3, 128, 64)])
+@pytest.mark.parametrize("M,B,N,K", [(1, 3, 40, 24), (9, 2, 130, 70), (70, 4, 64, 16), (200, 1, 33, 129), (5, 2, 70, 64), (2, 3, 33, 40), (1, 3, 40, 21), (8, 40, 128, 512), (40, 3, 128, 64), (100, 2, 70, 48), (64, 5, 96, 16), (33, 2, 33, 80)])
 @pytest.mark.parametrize("dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32)])
 def test_product_with_a_matrix_per_block_of_columns(M, B, N, K, dtype, out_dtype):
     from infinicore_infer_amd.kernels import ops
