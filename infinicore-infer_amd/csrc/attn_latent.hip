@@ -334,15 +334,18 @@ attn_latent_mfma_kernel(const bf16* __restrict__ qa, int qa_stride, bf16* __rest
         }
         __syncthreads();
         if (s + 1 < s_hi) fetch(s + 1);
-        lat_v16f sacc;
+        lat_v16f sacc, sacc2;                  // two chains of dependent products instead of one
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+        for (int r = 0; r < 16; ++r) sacc[r] = sacc2[r] = 0.f;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const lat_bf16x8 a = *reinterpret_cast<const lat_bf16x8*>(Ks + lq * PK + 16 * c + 8 * half);
             const lat_bf16x8 q = QLDS ? *reinterpret_cast<const lat_bf16x8*>(Qs + lq * PK + 16 * c + 8 * half) : qf[c];
-            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q, sacc, 0, 0, 0);
+            if (c & 1) sacc2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q, sacc2, 0, 0, 0);
+            else sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, q, sacc, 0, 0, 0);
         }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[r] += sacc2[r];
         if (kb + 31 > pos) {
 #pragma unroll
             for (int r = 0; r < 16; ++r)
