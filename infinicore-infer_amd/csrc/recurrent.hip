@@ -196,7 +196,7 @@ IC_EXPORT int ic_rglru_scan(const float* gates, const float* gate_bias, const fl
 //     S <- exp(neg_a[h] dt) S + dt B_g x_h^T   (S is N x P),   y_h = S^T C_g + D[h] x_h.
 // One block per (head, request, chunk).  Thread (grp, p) keeps column p of a run of NI rows of S in registers;
 // a token's B, C and x pass through LDS, the next token's are loaded while this one is computed.
-template <typename T, int NI>
+template <typename T, int NI, bool FULL>       // FULL: every thread owns exactly NI rows (N = NI * groups): no guards, 16-byte LDS reads
 __global__ void __launch_bounds__(256)
 ssm_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ dt_raw, int dt_stride,
                 const float* __restrict__ dt_bias, const float* __restrict__ neg_a, const float* __restrict__ Dw,
@@ -263,12 +263,25 @@ ssm_scan_kernel(const float* __restrict__ xbc, const T* __restrict__ dt_raw, int
         if (active) {
             const float dx = dt * xs[p];
             float acc = 0.f;
+            if (FULL) {
 #pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const int n = n0 + i;
-                if (i < ni && n < N) {
-                    s[i] = da * s[i] + Bs[n] * dx;
-                    acc += s[i] * Cs[n];
+                for (int i = 0; i < NI; i += 4) {
+                    const float4 b4 = *reinterpret_cast<const float4*>(Bs + n0 + i);
+                    const float4 c4 = *reinterpret_cast<const float4*>(Cs + n0 + i);
+                    s[i] = da * s[i] + b4.x * dx;
+                    s[i + 1] = da * s[i + 1] + b4.y * dx;
+                    s[i + 2] = da * s[i + 2] + b4.z * dx;
+                    s[i + 3] = da * s[i + 3] + b4.w * dx;
+                    acc += s[i] * c4.x + s[i + 1] * c4.y + s[i + 2] * c4.z + s[i + 3] * c4.w;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NI; ++i) {
+                    const int n = n0 + i;
+                    if (i < ni && n < N) {
+                        s[i] = da * s[i] + Bs[n] * dx;
+                        acc += s[i] * Cs[n];
+                    }
                 }
             }
             if (mode != 1) part[grp * P + p] = acc;
@@ -303,10 +316,18 @@ static int ssm_launch(int ni, dim3 grid, size_t lds, hipStream_t stream, const f
                       const float* dt_bias, const float* neg_a, const float* Dw, int heads, int P, int N, int G, float* y,
                       float* state, long long state_stride, const int* req_start, const int* state_slots, int mode,
                       int chunk_len, int max_chunks, float* scr_s, float* scr_a) {
+    const bool full = N % 4 == 0 && P % 4 == 0 && 256 % P == 0 && (256 / P) * ni == N;      // (multiples of 4 keep the LDS rows 16-byte aligned)
 #define IC_SSM(NI)                                                                                                      \
-    hipLaunchKernelGGL((ssm_scan_kernel<T, NI>), grid, dim3(256), lds, stream, xbc, (const T*)dt_raw, dt_stride, dt_bias, \
-                       neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots, mode, chunk_len,       \
-                       max_chunks, scr_s, scr_a)
+    do {                                                                                                                \
+    if (full && ni == NI)                                                                                               \
+        hipLaunchKernelGGL((ssm_scan_kernel<T, NI, true>), grid, dim3(256), lds, stream, xbc, (const T*)dt_raw, dt_stride, \
+                           dt_bias, neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots, mode,     \
+                           chunk_len, max_chunks, scr_s, scr_a);                                                         \
+    else                                                                                                                \
+        hipLaunchKernelGGL((ssm_scan_kernel<T, NI, false>), grid, dim3(256), lds, stream, xbc, (const T*)dt_raw, dt_stride, \
+                           dt_bias, neg_a, Dw, heads, P, N, G, y, state, state_stride, req_start, state_slots, mode,     \
+                           chunk_len, max_chunks, scr_s, scr_a);                                                         \
+    } while (0)
     if (ni <= 8) IC_SSM(8);
     else if (ni <= 16) IC_SSM(16);
     else if (ni <= 32) IC_SSM(32);
