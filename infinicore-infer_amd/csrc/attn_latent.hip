@@ -430,21 +430,22 @@ attn_latent_merge_kernel(const float* __restrict__ part_acc, const float* __rest
                          T* __restrict__ out, int out_stride, const int* __restrict__ row_list) {
     const int h = blockIdx.x % H, t = row_list ? row_list[blockIdx.x / H] : blockIdx.x / H;
     const size_t p0 = ((size_t)t * H + h) * n_split;
-    float m = -INFINITY;
-    for (int s = 0; s < n_split; ++s) m = fmaxf(m, part_ml[2 * (p0 + s)]);
-    float l = 0.f;
-    for (int s = 0; s < n_split; ++s) {
-        const float ms = part_ml[2 * (p0 + s)];
-        if (ms > -INFINITY) l += part_ml[2 * (p0 + s) + 1] * expf(ms - m);
+    __shared__ float wgt[64];                 // a split's share of the result: exp(m_s - m) / l
+    if (threadIdx.x < 64) {
+        const int sp = threadIdx.x;
+        const float ms = sp < n_split ? part_ml[2 * (p0 + sp)] : -INFINITY;
+        const float ls = sp < n_split ? part_ml[2 * (p0 + sp) + 1] : 0.f;
+        const float m = wave_max(ms);
+        const float e = ms > -INFINITY ? expf(ms - m) : 0.f;
+        const float l = wave_sum(ls * e);
+        wgt[sp] = e / l;
     }
-    const float inv = 1.0f / l;
+    __syncthreads();
     for (int j = threadIdx.x; j < R; j += blockDim.x) {
         float a = 0.f;
-        for (int s = 0; s < n_split; ++s) {
-            const float ms = part_ml[2 * (p0 + s)];
-            if (ms > -INFINITY) a += part_acc[(p0 + s) * R + j] * expf(ms - m);
-        }
-        out[(size_t)t * out_stride + (size_t)h * R + j] = from_f32<T>(a * inv);
+#pragma unroll 4
+        for (int sp = 0; sp < n_split; ++sp) a += part_acc[(p0 + sp) * R + j] * wgt[sp];     // (an empty split left zeros)
+        out[(size_t)t * out_stride + (size_t)h * R + j] = from_f32<T>(a);
     }
 }
 
