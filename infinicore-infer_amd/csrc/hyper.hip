@@ -216,7 +216,7 @@ IC_EXPORT int ic_hc_step(float* x, int S, int T, int d, const void* y, int y_dty
                          const float* out_w, const float* in_w, const float* norm_w, float eps, void* h, int h_dtype,
                          hipStream_t stream) {
     if (T <= 0) return IC_OK;
-    if (S <= 0 || S > kHcMaxStreams || d <= 0 || d > 16384 || (y && (!mix || !out_w)) || (in_w && !h)) return IC_ERR_ARG;
+    if (S <= 0 || S > kHcMaxStreams || d <= 0 || d > 16128 || (y && (!mix || !out_w)) || (in_w && !h)) return IC_ERR_ARG;
     const int yd = y ? y_dtype : (h_dtype == IC_F32 ? IC_F32 : IC_BF16);
     if (yd == IC_F32 && h_dtype == IC_F32) hc_launch<float, float>(x, S, T, d, y, mix, out_w, in_w, norm_w, eps, h, stream);
     else if (yd == IC_BF16 && h_dtype == IC_BF16) hc_launch<bf16, bf16>(x, S, T, d, y, mix, out_w, in_w, norm_w, eps, h, stream);

@@ -396,7 +396,7 @@ gated_group_norm_kernel(const float* __restrict__ y, const T* __restrict__ z, in
 IC_EXPORT int ic_gated_group_norm(const float* y, const void* z, int z_stride, int dtype, const float* w, int inner,
                                   int groups, float eps, void* out, int T, hipStream_t stream) {
     if (T <= 0) return IC_OK;
-    if (inner <= 0 || groups <= 0 || inner % groups || inner / groups > 16384) return IC_ERR_ARG;
+    if (inner <= 0 || groups <= 0 || inner % groups || inner / groups > 16128) return IC_ERR_ARG;
     const int gs = inner / groups;
     dim3 grid(T, groups), block(256);
     if (dtype == IC_F32)
